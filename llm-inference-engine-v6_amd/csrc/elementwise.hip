@@ -494,6 +494,40 @@ extern "C" int llme_swiglu(const void* gu, int in_dtype, void* out, int out_dtyp
     return launch_status();
 }
 
+// The same with the gate's activation chosen by a code: 0 silu, 1 relu, 2 gelu (tanh form).
+template <typename TI, typename TO>
+__global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int FF, int group, size_t total, int act) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / FF;
+    const int j = static_cast<int>(idx % FF);
+    const size_t base = t * 2 * static_cast<size_t>(FF) + static_cast<size_t>(j / group) * 2 * group + (j % group);
+    const float g = to_float(gu[base]);
+    const float u = to_float(gu[base + group]);
+    float a;
+    if (act == 1) a = fmaxf(g, 0.f);
+    else if (act == 2) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    else a = g / (1.0f + expf(-g));
+    out[idx] = from_float<TO>(a * u);
+}
+
+extern "C" int llme_gated_act(const void* gu, int in_dtype, void* out, int out_dtype, int T, int FF, int group, int act,
+                              hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (group <= 0 || FF % group != 0 || act < 0 || act > 2) return kErrBadArgument;
+    const size_t total = static_cast<size_t>(T) * FF;
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+#define LLME_GACT(TI, TO)                                                                        \
+    hipLaunchKernelGGL((gated_act_kernel<TI, TO>), grid, dim3(256), 0, stream,                   \
+                       static_cast<const TI*>(gu), static_cast<TO*>(out), FF, group, total, act)
+    if (in_dtype == kF32 && out_dtype == kF32) LLME_GACT(float, float);
+    else if (in_dtype == kF32 && out_dtype == kBF16) LLME_GACT(float, bf16);
+    else if (in_dtype == kBF16 && out_dtype == kBF16) LLME_GACT(bf16, bf16);
+    else return kErrBadArgument;
+#undef LLME_GACT
+    return launch_status();
+}
+
 // zero_input (with write_cache): qkv is all zeros afterwards (by the kernel itself where one thread
 // reads each value once, else by the clearing kernel behind it).
 extern "C" int llme_rope_kv_write(float* qkv, const float* cos_t, const float* sin_t,

@@ -1,0 +1,442 @@
+// Mixers that carry a state of fixed size from token to token: short causal convolutions, the gated
+// diagonal recurrence (RG-LRU) and the gated delta rule. Everything that enters a recurrence, and the
+// state itself, is 32-bit; only weights may be stored in bfloat16 (they are widened exactly).
+//
+// A step is a flat batch of rows; request s owns rows q_start[s] .. q_start[s + 1] - 1, which continue
+// what its slot (slots[s]) of every state tensor holds. Inputs are column ranges of wider 32-bit
+// buffers (a fused projection's output), so every matrix comes with its leading dimension.
+#include "common.h"
+
+namespace llme {
+
+constexpr int kMaxTaps = 16;
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float gelu_tanhf_(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// ---------------------------------------------------------------------------------
+// out[t, c] = act(bias[c] + sum_j w[c, j] * x[t - (K - 1 - j), c]) with x = in + in_bias (a bias of the product in
+// front, null for none); rows before the request's first row of this step come from the slot's tail [K - 1, C]
+// (oldest first; zero for a new request: what lies before a sequence's start counts as zero, bias and all).
+__global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ in, int ld_in, const float* __restrict__ w,
+                                                         const float* __restrict__ bias, const float* __restrict__ in_bias,
+                                                         const float* __restrict__ tail, const int* __restrict__ seq_idx, const int* __restrict__ q_start,
+                                                         const int* __restrict__ slots, float* __restrict__ out, int ld_out,
+                                                         int C, int K, int act) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int s = seq_idx[t];
+    const int first = q_start[s];
+    const float* tl = tail + static_cast<size_t>(slots[s]) * (K - 1) * C;
+    float acc = bias ? bias[c] : 0.f;
+    const float ib = in_bias ? in_bias[c] : 0.f;
+    for (int j = 0; j < K; ++j) {
+        const int r = t - (K - 1 - j);
+        const float x = r >= first ? in[static_cast<size_t>(r) * ld_in + c] + ib
+                                   : tl[static_cast<size_t>(K - 1 + (r - first)) * C + c];
+        acc += w[static_cast<size_t>(c) * K + j] * x;
+    }
+    out[static_cast<size_t>(t) * ld_out + c] = act == 1 ? siluf_(acc) : acc;
+}
+
+// The slot's tail after the step: the last K - 1 inputs of the request, from this step's rows and, where the
+// step brought fewer, from the old tail.
+__global__ __launch_bounds__(256) void conv_tail_kernel(const float* __restrict__ in, int ld_in,
+                                                        const float* __restrict__ in_bias, float* __restrict__ tail,
+                                                        const int* __restrict__ q_start, const int* __restrict__ slots,
+                                                        int C, int K) {
+    const int s = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int first = q_start[s], n = q_start[s + 1] - first;
+    float* tl = tail + static_cast<size_t>(slots[s]) * (K - 1) * C;
+    float keep[kMaxTaps];
+    const float ib = in_bias ? in_bias[c] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+        if (i >= K - 1) break;
+        const int rel = n - (K - 1) + i;            // row of the new tail's entry i, counted from the step's first
+        keep[i] = rel >= 0 ? in[static_cast<size_t>(first + rel) * ld_in + c] + ib : tl[static_cast<size_t>(K - 1 + rel) * C + c];
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+        if (i >= K - 1) break;
+        tl[static_cast<size_t>(i) * C + c] = keep[i];
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// RG-LRU gates. u [T, width] in blocks of bw channels; per block b two maps [bw, bw] ([out, in]):
+//   r = sigmoid(Ra_b u_b + ba), i = sigmoid(Ri_b u_b + bi), a = exp(-c r softplus(lam)),
+//   decay[t, ch] = a,  drive[t, ch] = sqrt(1 - a^2) i u.
+// A workgroup makes 16 rows x 64 channels of one block, stepping through the block's inputs in slabs of 32.
+template <typename TW>
+__global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restrict__ u, int ld_u, const TW* __restrict__ ra,
+                                                          const float* __restrict__ rab, const TW* __restrict__ ri,
+                                                          const float* __restrict__ rib, const float* __restrict__ lam,
+                                                          float* __restrict__ decay, float* __restrict__ drive, int T,
+                                                          int width, int bw, float c_rate) {
+    constexpr int TM = 16, TN = 64, TK = 32;
+    __shared__ float us[TM][TK + 1];
+    __shared__ float was[TN][TK + 1];
+    __shared__ float wis[TN][TK + 1];
+    const int tiles_n = (bw + TN - 1) / TN;
+    const int b = blockIdx.x / tiles_n;
+    const int n0 = (blockIdx.x % tiles_n) * TN;
+    const int t0 = blockIdx.y * TM;
+    const int tid = threadIdx.x;
+    const int tm = tid / 16;            // row of the tile
+    const int tn = tid % 16;            // channels tn, tn + 16, tn + 32, tn + 48
+    float accr[4] = {0.f, 0.f, 0.f, 0.f}, acci[4] = {0.f, 0.f, 0.f, 0.f};
+    const TW* ra_b = ra + static_cast<size_t>(b) * bw * bw;
+    const TW* ri_b = ri + static_cast<size_t>(b) * bw * bw;
+    for (int k0 = 0; k0 < bw; k0 += TK) {
+        for (int e = tid; e < TM * TK; e += 256) {
+            const int r = e / TK, k = e % TK;
+            us[r][k] = (t0 + r < T && k0 + k < bw) ? u[static_cast<size_t>(t0 + r) * ld_u + b * bw + k0 + k] : 0.f;
+        }
+        for (int e = tid; e < TN * TK; e += 256) {
+            const int o = e / TK, k = e % TK;
+            const bool ok = n0 + o < bw && k0 + k < bw;
+            was[o][k] = ok ? to_float(ra_b[static_cast<size_t>(n0 + o) * bw + k0 + k]) : 0.f;
+            wis[o][k] = ok ? to_float(ri_b[static_cast<size_t>(n0 + o) * bw + k0 + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int k = 0; k < TK; ++k) {
+            const float x = us[tm][k];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                accr[j] += was[tn + 16 * j][k] * x;
+                acci[j] += wis[tn + 16 * j][k] * x;
+            }
+        }
+        __syncthreads();
+    }
+    const int t = t0 + tm;
+    if (t >= T) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int o = n0 + tn + 16 * j;
+        if (o >= bw) continue;
+        const int ch = b * bw + o;
+        const float r = sigmoidf_(accr[j] + rab[ch]);
+        const float g = sigmoidf_(acci[j] + rib[ch]);
+        const float log_a = -c_rate * r * softplusf_(lam[ch]);
+        const float a = expf(log_a);
+        const float x = u[static_cast<size_t>(t) * ld_u + ch];
+        decay[static_cast<size_t>(t) * width + ch] = a;
+        drive[static_cast<size_t>(t) * width + ch] = sqrtf(-expm1f(2.0f * log_a)) * (g * x);
+    }
+}
+
+// s_t = decay_t s_(t-1) + drive_t per request and channel, from the slot's state; out[t] = s_t * gelu_tanh(y[t] + yb)
+// in the activation type. A thread walks one channel of one request through the step's rows.
+template <typename TO>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(const float* __restrict__ decay, const float* __restrict__ drive,
+                                                         const float* __restrict__ y, int ld_y, const float* __restrict__ yb,
+                                                         float* __restrict__ state, const int* __restrict__ q_start,
+                                                         const int* __restrict__ slots, TO* __restrict__ out, int ld_out,
+                                                         int width) {
+    const int s = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= width) return;
+    const int first = q_start[s], last = q_start[s + 1];
+    float* st = state + static_cast<size_t>(slots[s]) * width + c;
+    float h = *st;
+    const float bias = yb ? yb[c] : 0.f;
+    for (int t = first; t < last; ++t) {
+        const size_t at = static_cast<size_t>(t) * width + c;
+        h = decay[at] * h + drive[at];
+        out[static_cast<size_t>(t) * ld_out + c] = from_float<TO>(h * gelu_tanhf_(y[static_cast<size_t>(t) * ld_y + c] + bias));
+    }
+    *st = h;
+}
+
+// ---------------------------------------------------------------------------------
+// x <- x / sqrt(sum(x^2) + eps) * scale over every head of `dim` entries, in place; heads [0, n_a) scale by
+// scale_a, heads [n_a, n_a + n_b) by scale_b (queries and keys lie side by side). One wavefront per (row, head).
+__global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, int ld, int T, int n_a, int n_b, int dim,
+                                                         float scale_a, float scale_b, float eps) {
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int item = blockIdx.x * 4 + wave;
+    if (item >= T * (n_a + n_b)) return;
+    const int t = item / (n_a + n_b), h = item % (n_a + n_b);
+    float* p = x + static_cast<size_t>(t) * ld + static_cast<size_t>(h) * dim;
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += kWave) ss += p[i] * p[i];
+    ss = wave_sum(ss);
+    const float f = (h < n_a ? scale_a : scale_b) / sqrtf(ss + eps);
+    for (int i = lane; i < dim; i += kWave) p[i] *= f;
+}
+
+// beta[t, h] = sigmoid(b[t, h]);
+// per channel: decay[t, h, d] = exp(-exp(A_log[h]) softplus(sum_r a2[h dim + d, r] a1[t, r] + dt_bias[h dim + d]))
+// per head:    decay[t, h]    = exp(-exp(A_log[h]) softplus(a[t, h] + dt_bias[h]))
+template <typename TW>
+__global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restrict__ b_in, int ld_b, const float* __restrict__ a_in,
+                                                          int ld_a, const TW* __restrict__ a2, int rank,
+                                                          const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                                                          float* __restrict__ beta, float* __restrict__ decay, int T, int heads,
+                                                          int dim, int per_channel) {
+    const int t = blockIdx.y;
+    const int n_dec = per_channel ? heads * dim : heads;
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e < heads) beta[static_cast<size_t>(t) * heads + e] = sigmoidf_(b_in[static_cast<size_t>(t) * ld_b + e]);
+    if (e >= n_dec) return;
+    const int h = per_channel ? e / dim : e;
+    float z;
+    if (per_channel) {
+        z = 0.f;
+        const float* lo = a_in + static_cast<size_t>(t) * ld_a;
+        const TW* row = a2 + static_cast<size_t>(e) * rank;
+        for (int r = 0; r < rank; ++r) z += to_float(row[r]) * lo[r];
+    } else {
+        z = a_in[static_cast<size_t>(t) * ld_a + e];
+    }
+    z += dt_bias[e];
+    decay[static_cast<size_t>(t) * n_dec + e] = expf(-expf(A_log[h]) * softplusf_(z));
+}
+
+// The delta rule. State M [dim, vdim] per request and head (32-bit, in the request's slot). Per token:
+//   M <- g * M (g per key channel or one per head);  w = beta (v - M^T k);  M <- M + k w^T;  o = M^T q.
+// The columns of M do not depend on each other: four lanes share a column (lane l holds the key channels
+// l, l + 4, ...), a workgroup of 256 threads owns 64 columns of one head of one request and walks the
+// request's rows in order. R = channels per lane.
+template <int R, bool PER_CHANNEL>
+__global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int ld, int q_col, int k_col, int v_col,
+                                                         const float* __restrict__ beta, const float* __restrict__ decay,
+                                                         float* __restrict__ state, const int* __restrict__ q_start,
+                                                         const int* __restrict__ slots, float* __restrict__ o, int heads,
+                                                         int kv_heads, int dim, int vdim) {
+    const int s = blockIdx.z, h = blockIdx.y;
+    const int col = blockIdx.x * 64 + threadIdx.x / 4;
+    const int l = threadIdx.x % 4;
+    const bool live = col < vdim;
+    const int kvh = h / (heads / kv_heads);
+    const int first = q_start[s], last = q_start[s + 1];
+    float* M = state + (static_cast<size_t>(slots[s]) * heads + h) * dim * vdim;
+    float m[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int d = l + 4 * i;
+        m[i] = (live && d < dim) ? M[static_cast<size_t>(d) * vdim + col] : 0.f;
+    }
+    const int n_dec = PER_CHANNEL ? heads * dim : heads;
+    for (int t = first; t < last; ++t) {
+        const float* row = qkv + static_cast<size_t>(t) * ld;
+        const float* kp = row + k_col + kvh * dim;
+        const float* qp = row + q_col + kvh * dim;
+        const float* gp = decay + static_cast<size_t>(t) * n_dec + (PER_CHANNEL ? h * dim : h);
+        const float bt = beta[static_cast<size_t>(t) * heads + h];
+        const float vv = live ? row[v_col + h * vdim + col] : 0.f;
+        float kk[R], qq[R];
+        const float g_head = PER_CHANNEL ? 1.f : gp[0];
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int d = l + 4 * i;
+            const bool in = d < dim;
+            kk[i] = in ? kp[d] : 0.f;
+            qq[i] = in ? qp[d] : 0.f;
+            const float g = PER_CHANNEL ? (in ? gp[d] : 0.f) : g_head;
+            m[i] *= g;
+            dot += m[i] * kk[i];
+        }
+        dot += __shfl_xor(dot, 1, kWave);
+        dot += __shfl_xor(dot, 2, kWave);
+        const float w = bt * (vv - dot);
+        float read = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            m[i] += kk[i] * w;
+            read += m[i] * qq[i];
+        }
+        read += __shfl_xor(read, 1, kWave);
+        read += __shfl_xor(read, 2, kWave);
+        if (live && l == 0) o[static_cast<size_t>(t) * heads * vdim + h * vdim + col] = read;
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int d = l + 4 * i;
+        if (live && d < dim) M[static_cast<size_t>(d) * vdim + col] = m[i];
+    }
+}
+
+// out[t, h, j] = scale * o[t, h, j] / sqrt(mean_j o^2 + eps) * w[j] * gate, in the activation type.
+//   gate 0: sigmoid(sum_r g2[h vdim + j, r] g1[t, r]);  gate 1: silu(g[t, h vdim + j])
+// One wavefront per (row, head).
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                              const float* __restrict__ g_in, int ld_g, const TW* __restrict__ g2,
+                                                              int rank, int gate, TO* __restrict__ out, int ld_out, int T, int heads,
+                                                              int vdim, float eps, float scale) {
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int item = blockIdx.x * 4 + wave;
+    if (item >= T * heads) return;
+    const int t = item / heads, h = item % heads;
+    const float* p = o + (static_cast<size_t>(t) * heads + h) * vdim;
+    float ss = 0.f;
+    for (int j = lane; j < vdim; j += kWave) ss += p[j] * p[j];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(vdim) + eps);
+    const float* gi = g_in + static_cast<size_t>(t) * ld_g;
+    for (int j = lane; j < vdim; j += kWave) {
+        float z;
+        if (gate == 0) {
+            z = 0.f;
+            const TW* row = g2 + static_cast<size_t>(h * vdim + j) * rank;
+            for (int r = 0; r < rank; ++r) z += to_float(row[r]) * gi[r];
+            z = sigmoidf_(z);
+        } else {
+            z = siluf_(gi[h * vdim + j]);
+        }
+        out[static_cast<size_t>(t) * ld_out + h * vdim + j] = from_float<TO>(scale * ((p[j] * inv) * w[j] * z));
+    }
+}
+
+}  // namespace llme
+
+using namespace llme;
+
+#define LLME_BY_W(dt, CALL)                                  \
+    if ((dt) == kF32) { using TW = float; CALL; }            \
+    else if ((dt) == kBF16) { using TW = bf16; CALL; }       \
+    else return kErrBadArgument;
+
+// in [T, ld_in] 32-bit; w [C, K], bias [C] or null (w_dtype); tail [slots, K - 1, C] 32-bit; out [T, ld_out] 32-bit.
+// update_tail: after the convolution the slots' tails are moved on by the step's rows.
+extern "C" int llme_short_conv(const void* in, int ld_in, const void* w, const void* bias, const void* in_bias, void* tail,
+                               const void* seq_idx, const void* q_start, const void* slots, void* out, int ld_out, int T,
+                               int n_seq, int C, int K, int act, int update_tail, hipStream_t stream) {
+    if (T <= 0 || C <= 0) return 0;
+    if (K < 1 || K > kMaxTaps) return kErrUnsupported;
+    const dim3 grid((C + 255) / 256, T);
+    short_conv_kernel<<<grid, 256, 0, stream>>>(
+        static_cast<const float*>(in), ld_in, static_cast<const float*>(w), static_cast<const float*>(bias),
+        static_cast<const float*>(in_bias), static_cast<const float*>(tail), static_cast<const int*>(seq_idx), static_cast<const int*>(q_start),
+        static_cast<const int*>(slots), static_cast<float*>(out), ld_out, C, K, act);
+    if (update_tail && K > 1)
+        conv_tail_kernel<<<dim3((C + 255) / 256, n_seq), 256, 0, stream>>>(
+            static_cast<const float*>(in), ld_in, static_cast<const float*>(in_bias), static_cast<float*>(tail),
+            static_cast<const int*>(q_start),
+            static_cast<const int*>(slots), C, K);
+    return launch_status();
+}
+
+extern "C" int llme_rglru_gates(const void* u, int ld_u, const void* ra, const void* rab, const void* ri, const void* rib,
+                                const void* lam, int w_dtype, void* decay, void* drive, int T, int width, int blocks,
+                                float c_rate, hipStream_t stream) {
+    if (T <= 0 || width <= 0) return 0;
+    if (blocks <= 0 || width % blocks) return kErrBadArgument;
+    const int bw = width / blocks;
+    const dim3 grid(blocks * ((bw + 63) / 64), (T + 15) / 16);
+    LLME_BY_W(w_dtype, (rglru_gates_kernel<TW><<<grid, 256, 0, stream>>>(
+        static_cast<const float*>(u), ld_u, static_cast<const TW*>(ra), static_cast<const float*>(rab),
+        static_cast<const TW*>(ri), static_cast<const float*>(rib), static_cast<const float*>(lam), static_cast<float*>(decay),
+        static_cast<float*>(drive), T, width, bw, c_rate)));
+    return launch_status();
+}
+
+extern "C" int llme_rglru_scan(const void* decay, const void* drive, const void* y, int ld_y, const void* yb,
+                               void* state, const void* q_start, const void* slots, void* out, int out_dtype, int ld_out,
+                               int n_seq, int width, hipStream_t stream) {
+    if (n_seq <= 0 || width <= 0) return 0;
+    const dim3 grid((width + 255) / 256, n_seq);
+#define LLME_SCAN(TO_)                                                                                                   \
+    rglru_scan_kernel<TO_><<<grid, 256, 0, stream>>>(                                                                    \
+        static_cast<const float*>(decay), static_cast<const float*>(drive), static_cast<const float*>(y), ld_y,          \
+        static_cast<const float*>(yb), static_cast<float*>(state), static_cast<const int*>(q_start),                     \
+        static_cast<const int*>(slots), static_cast<TO_*>(out), ld_out, width)
+    switch (out_dtype) {
+        case kF32: LLME_SCAN(float); break;
+        case kBF16: LLME_SCAN(bf16); break;
+        default: return kErrBadArgument;
+    }
+#undef LLME_SCAN
+    return launch_status();
+}
+
+extern "C" int llme_unit_heads(void* x, int ld, int T, int n_a, int n_b, int dim, float scale_a, float scale_b, float eps,
+                               hipStream_t stream) {
+    const long items = static_cast<long>(T) * (n_a + n_b);
+    if (items <= 0 || dim <= 0) return 0;
+    unit_heads_kernel<<<static_cast<int>((items + 3) / 4), 256, 0, stream>>>(static_cast<float*>(x), ld, T, n_a, n_b, dim,
+                                                                            scale_a, scale_b, eps);
+    return launch_status();
+}
+
+extern "C" int llme_delta_gates(const void* b_in, int ld_b, const void* a_in, int ld_a, const void* a2, int rank,
+                                const void* A_log, const void* dt_bias, int w_dtype, void* beta, void* decay, int T, int heads,
+                                int dim, int per_channel, hipStream_t stream) {
+    if (T <= 0 || heads <= 0) return 0;
+    const int n = per_channel ? heads * dim : heads;
+    const dim3 grid(((n > heads ? n : heads) + 255) / 256, T);
+    LLME_BY_W(w_dtype, (delta_gates_kernel<TW><<<grid, 256, 0, stream>>>(
+        static_cast<const float*>(b_in), ld_b, static_cast<const float*>(a_in), ld_a, static_cast<const TW*>(a2), rank,
+        static_cast<const float*>(A_log), static_cast<const float*>(dt_bias), static_cast<float*>(beta),
+        static_cast<float*>(decay), T, heads, dim, per_channel)));
+    return launch_status();
+}
+
+template <int R>
+static void launch_delta_rule(bool per_channel, dim3 grid, hipStream_t stream, const float* qkv, int ld, int q_col, int k_col,
+                              int v_col, const float* beta, const float* decay, float* state, const int* q_start,
+                              const int* slots, float* o, int heads, int kv_heads, int dim, int vdim) {
+    if (per_channel)
+        delta_rule_kernel<R, true><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
+                                                             heads, kv_heads, dim, vdim);
+    else
+        delta_rule_kernel<R, false><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
+                                                              heads, kv_heads, dim, vdim);
+}
+
+// qkv [T, ld] 32-bit with unit q at q_col, unit k at k_col (kv_heads x dim each) and v at v_col (heads x vdim);
+// beta [T, heads]; decay [T, heads, dim] or [T, heads]; state [slots, heads, dim, vdim]; o [T, heads, vdim] 32-bit.
+extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, int v_col, const void* beta, const void* decay,
+                               int per_channel, void* state, const void* q_start, const void* slots, void* o, int n_seq,
+                               int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
+    if (n_seq <= 0 || heads <= 0) return 0;
+    if (kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return kErrBadArgument;
+    if (dim > 256) return kErrUnsupported;
+    const dim3 grid((vdim + 63) / 64, heads, n_seq);
+#define LLME_DELTA(R_)                                                                                                   \
+    launch_delta_rule<R_>(per_channel != 0, grid, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col,      \
+                          static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state), \
+                          static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(o), heads, \
+                          kv_heads, dim, vdim)
+    if (dim <= 32) LLME_DELTA(8);
+    else if (dim <= 64) LLME_DELTA(16);
+    else if (dim <= 128) LLME_DELTA(32);
+    else LLME_DELTA(64);
+#undef LLME_DELTA
+    return launch_status();
+}
+
+extern "C" int llme_gated_head_norm(const void* o, const void* w, const void* g_in, int ld_g, const void* g2, int rank, int gate,
+                                    int w_dtype, void* out, int out_dtype, int ld_out, int T, int heads, int vdim, float eps,
+                                    float scale, hipStream_t stream) {
+    const long items = static_cast<long>(T) * heads;
+    if (items <= 0 || vdim <= 0) return 0;
+    const int grid = static_cast<int>((items + 3) / 4);
+#define LLME_GHN(TW_, TO_)                                                                                               \
+    gated_head_norm_kernel<TW_, TO_><<<grid, 256, 0, stream>>>(                                                          \
+        static_cast<const float*>(o), static_cast<const float*>(w), static_cast<const float*>(g_in), ld_g,               \
+        static_cast<const TW_*>(g2), rank, gate, static_cast<TO_*>(out), ld_out, T, heads, vdim, eps, scale)
+    switch (w_dtype * 2 + out_dtype) {
+        case 0: LLME_GHN(float, float); break;
+        case 1: LLME_GHN(float, bf16); break;
+        case 2: LLME_GHN(bf16, float); break;
+        case 3: LLME_GHN(bf16, bf16); break;
+        default: return kErrBadArgument;
+    }
+#undef LLME_GHN
+    return launch_status();
+}
+
+LLME_LOAD_ENTRY(recurrent)

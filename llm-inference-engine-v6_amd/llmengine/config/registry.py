@@ -36,9 +36,11 @@ def known_architectures() -> list[str]:
 
 def architecture_name(cfg: Mapping[str, Any]) -> str:
     archs = cfg.get("architectures")
+    if archs is None and isinstance(cfg.get("architecture"), str):
+        return cfg["architecture"]          # (some designs name theirs under a key of its own)
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json: key 'architectures' must be a non-empty list of names; "
-                          f"known architectures: {known_architectures()}")
+        raise ConfigError("config.json: key 'architectures' must be a non-empty list of names (or 'architecture' "
+                          f"one name); known architectures: {known_architectures()}")
     return archs[0]
 
 

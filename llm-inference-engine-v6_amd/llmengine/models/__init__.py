@@ -1,4 +1,5 @@
 from .model import DecoderModel, LayerCall
 from . import llama  # registers "LlamaForCausalLM"
+from . import rilonex  # registers "Rilonex"
 
-__all__ = ["DecoderModel", "LayerCall", "llama"]
+__all__ = ["DecoderModel", "LayerCall", "llama", "rilonex"]

@@ -13,6 +13,7 @@ from dataclasses import dataclass
 
 import torch
 
+from .. import ops
 from ..parts.base import Block, CacheSpec, Head, Norm, Part, TokenEmbedding
 
 
@@ -31,8 +32,11 @@ class DecoderModel(Part):
     graph_safe = True
 
     def __init__(self, config, embedding: TokenEmbedding, layers: list[Block], final_norm: Norm,
-                 head: Head, schedule: list[LayerCall] | None = None, names: dict | None = None):
+                 head: Head, schedule: list[LayerCall] | None = None, names: dict | None = None, streams: int = 0):
         self.config = config
+        # streams > 0: the residual is kept as that many streams [streams, T, H] (blocks that know how read and
+        # write them); every stream starts as the embedding, and the final norm reads their sum
+        self.streams = int(streams)
         self.embedding, self.layers, self.final_norm, self.head = embedding, list(layers), final_norm, head
         self.schedule = list(schedule) if schedule is not None else [LayerCall(i) for i in range(len(layers))]
         for call in self.schedule:
@@ -48,7 +52,8 @@ class DecoderModel(Part):
         n = self.names
         out: dict[str, Part] = {n["embedding"]: self.embedding}
         for i, layer in enumerate(self.layers):
-            out[f"{n['layers']}.{i}"] = layer
+            # ("model.layers" names layer 3 "model.layers.3"; a pattern with "{}" puts the number where it says)
+            out[n["layers"].format(i) if "{}" in n["layers"] else f"{n['layers']}.{i}"] = layer
         out[n["final_norm"]] = self.final_norm
         out[n["head"]] = self.head
         return out
@@ -105,15 +110,31 @@ class DecoderModel(Part):
         """Runs the step's tokens through the schedule; returns 32-bit logits
         [len(logit_rows), vocab] for the wanted rows (None if none is wanted)."""
         T = step.num_tokens
-        h = step.buffer("model.hidden", (T, self.hidden_size), torch.float32)
-        self.embedding.forward(step.tokens, h, step)
+        if self.streams:
+            h = step.buffer("model.hidden", (self.streams, T, self.hidden_size), torch.float32)
+            self.embedding.forward(step.tokens, h[0], step)
+            ops.streams_spread(h)
+        else:
+            h = step.buffer("model.hidden", (T, self.hidden_size), torch.float32)
+            self.embedding.forward(step.tokens, h, step)
         for call in self.schedule:
             self.layers[call.layer].forward(h, step, caches[call.cache_id], call.write_cache)
         if logit_rows is None or logit_rows.shape[0] == 0:
             return None
         R = logit_rows.shape[0]
         logits = step.buffer("model.logits", (R, self.vocab_size), torch.float32)
-        if self.head.fuses_norm(h, self.final_norm, R, step):
+        if self.streams:
+            # the sum of the streams and the final norm in one kernel, at the wanted rows only
+            x = step.buffer("model.head_in", (R, self.hidden_size), step.act_dtype)
+            rms = self.final_norm.fused_rms()
+            if rms is not None:
+                ops.streams_read_norm(h, None, rms[0], rms[1], x, rows=logit_rows)
+            else:
+                total = step.buffer("model.stream_sum", (R, self.hidden_size), torch.float32)
+                ops.streams_read_norm(h, None, None, 0.0, total, rows=logit_rows)
+                self.final_norm.forward(total, x)
+            self.head.forward(x, logits, step)
+        elif self.head.fuses_norm(h, self.final_norm, R, step):
             self.head.forward_normed_rows(h, logit_rows, self.final_norm, logits, step)
         else:
             x = step.buffer("model.head_in", (R, self.hidden_size), step.act_dtype)

@@ -7,8 +7,14 @@ from .embedding import Embedding, OutputHead
 from .mlp import GatedMLP
 from .attention import Attention
 from .block import PreNormBlock
+from .projected import ParallelMixer, ProjectedMixer
+from .rglru import RGLRU
+from .delta import GatedDeltaRule
+from .sigmoid_attention import SigmoidAttention
+from .hyper import HyperConnectionBlock
 
 __all__ = ["PAGE", "Block", "CacheSpec", "FeedForward", "LayerCache", "Mixer", "Norm", "ParamSpec", "Part",
            "Placement", "PositionEncoding", "TokenEmbedding", "Head", "LayerSpec", "PartChoice", "build_layer", "make_part",
            "register_part", "registered", "RMSNorm", "RotaryEmbedding", "inverse_frequencies", "Embedding",
-           "OutputHead", "GatedMLP", "Attention", "PreNormBlock"]
+           "OutputHead", "GatedMLP", "Attention", "PreNormBlock", "ParallelMixer", "ProjectedMixer", "RGLRU", "GatedDeltaRule",
+           "SigmoidAttention", "HyperConnectionBlock"]

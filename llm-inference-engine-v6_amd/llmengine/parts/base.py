@@ -35,9 +35,18 @@ import torch
 @dataclass(frozen=True)
 class ParamSpec:
     """A tensor a part reads from the checkpoint: its exact shape there, and how a
-    random model fills it ("linear": N(0, std); "norm": N(mean, std) around one)."""
-    shape: tuple[int, ...]
+    random model fills it ("linear": N(0, std); "norm": N(mean, std) around one; "identity": the
+    unit matrix plus N(0, std); "taps": N(0, 1/2), for the few taps of a short convolution). A
+    dimension that only the checkpoint knows (a rank no configuration names) is None: any size
+    fits, and the part reads it off the tensor when it loads."""
+    shape: tuple[int | None, ...]
     init: str = "linear"
+
+
+def join_name(prefix: str, local: str) -> str:
+    """The full name of a part's tensor: the part's prefix (which ends in a dot) and the local
+    name; a part whose only tensor carries the part's own name calls it ""."""
+    return prefix + local if local else prefix.rstrip(".")
 
 
 @dataclass(frozen=True)
@@ -124,19 +133,19 @@ class Part:
 
     # ---- walking a tree of parts ----
     def named_specs(self, prefix: str = "") -> dict[str, ParamSpec]:
-        out = {prefix + k: v for k, v in self.param_specs().items()}
+        out = {join_name(prefix, k): v for k, v in self.param_specs().items()}
         for name, child in self.children().items():
             out.update(child.named_specs(f"{prefix}{name}."))
         return out
 
     def named_ignored(self, prefix: str = "") -> set[str]:
-        out = {prefix + k for k in self.ignored_names()}
+        out = {join_name(prefix, k) for k in self.ignored_names()}
         for name, child in self.children().items():
             out |= child.named_ignored(f"{prefix}{name}.")
         return out
 
     def named_aliases(self, prefix: str = "") -> dict[str, str]:
-        out = {prefix + a: prefix + t for a, t in self.aliases().items()}
+        out = {join_name(prefix, a): join_name(prefix, t) for a, t in self.aliases().items()}
         for name, child in self.children().items():
             out.update(child.named_aliases(f"{prefix}{name}."))
         return out
@@ -145,7 +154,7 @@ class Part:
         return bool(self.graph_safe) and all(c.tree_graph_safe() for c in self.children().values())
 
     def load_tree(self, get: Getter, placement: Placement, prefix: str = "") -> None:
-        self.load_params(lambda local: get(prefix + local), placement)
+        self.load_params(lambda local: get(join_name(prefix, local)), placement)
         for name, child in self.children().items():
             child.load_tree(get, placement, f"{prefix}{name}.")
 

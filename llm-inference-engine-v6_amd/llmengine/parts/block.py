@@ -13,7 +13,7 @@ from .registry import register_part
 class PreNormBlock(Block):
     graph_safe = True
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm,
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm, ffn_norm: Norm | None,
                  names: dict | None = None):
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
@@ -25,8 +25,10 @@ class PreNormBlock(Block):
 
     def children(self):
         n = self.names
-        return {n["mixer_norm"]: self.mixer_norm, n["mixer"]: self.mixer,
-                n["ffn_norm"]: self.ffn_norm, n["feed_forward"]: self.feed_forward}
+        out = {n["mixer_norm"]: self.mixer_norm, n["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out.update({n["ffn_norm"]: self.ffn_norm, n["feed_forward"]: self.feed_forward})
+        return out
 
     def forward(self, h, step, cache, write_cache=True):
         T, H = h.shape
@@ -36,6 +38,8 @@ class PreNormBlock(Block):
         else:
             self.mixer_norm.forward(h, x)
             self.mixer.forward(x, step, cache, h, True, write_cache)
+        if self.feed_forward is None:
+            return
         if self.feed_forward.fuses_norm(h, self.ffn_norm, step):
             self.feed_forward.forward(h, step, h, True, pre_norm=self.ffn_norm)
         else:

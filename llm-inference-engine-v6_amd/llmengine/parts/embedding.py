@@ -16,16 +16,17 @@ from .registry import register_part
 class Embedding(TokenEmbedding):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, tensor: str = "weight"):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tensor = tensor            # the local name of the table ("": the part's own name)
         self.weight: torch.Tensor | None = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+        return {self.tensor: ParamSpec((self.vocab_size, self.hidden_size), "linear")}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
         # (a tied head reads the table as a weight matrix: the gather takes either layout)
-        self.weight = placement.place_matrix(get("weight"))
+        self.weight = placement.place_matrix(get(self.tensor))
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor, step=None) -> None:
         ops.embed_gather(self.weight, tokens, out)
@@ -34,19 +35,20 @@ class Embedding(TokenEmbedding):
 class OutputHead(Head):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None, tensor: str = "weight"):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to
+        self.tensor = tensor
         self._weight: torch.Tensor | None = None
 
     def param_specs(self):
         if self.tied_to is not None:
             return {}
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+        return {self.tensor: ParamSpec((self.vocab_size, self.hidden_size), "linear")}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
         if self.tied_to is None:
-            self._weight = placement.place_matrix(get("weight"))
+            self._weight = placement.place_matrix(get(self.tensor))
 
     @property
     def weight(self) -> torch.Tensor:

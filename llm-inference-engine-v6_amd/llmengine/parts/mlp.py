@@ -1,5 +1,5 @@
-"""SiLU-gated feed-forward: down( silu(gate(x)) * up(x) ), no biases
-(src/engine.cpp:213-217, src/kernels.cpp:26-31).
+"""Gated feed-forward: down( act(gate(x)) * up(x) ), no biases; act is SiLU
+(src/engine.cpp:213-217, src/kernels.cpp:26-31) unless the model names another.
 
 Gate and up rows are stored interleaved in groups of 16 in one matrix, so that one
 product yields both and a 16-column group of its output holds the gate and the up
@@ -17,32 +17,38 @@ from .registry import register_part
 class GatedMLP(FeedForward):
     graph_safe = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", names: dict | None = None):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"gated_mlp: activation {activation!r} is none of {sorted(ops.GATE_ACTIVATIONS)}")
+        self.activation = activation
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        if names:
+            self.names.update(names)
         self.group = 16 if self.intermediate_size % 16 == 0 else self.intermediate_size
         self.w_gate_up: torch.Tensor | None = None
         self.w_down: torch.Tensor | None = None
 
     def param_specs(self):
         H, FF = self.hidden_size, self.intermediate_size
-        return {"gate_proj.weight": ParamSpec((FF, H)), "up_proj.weight": ParamSpec((FF, H)),
-                "down_proj.weight": ParamSpec((H, FF))}
+        n = self.names
+        return {n["gate"]: ParamSpec((FF, H)), n["up"]: ParamSpec((FF, H)), n["down"]: ParamSpec((H, FF))}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
         H, FF, g = self.hidden_size, self.intermediate_size, self.group
-        gate, up = get("gate_proj.weight"), get("up_proj.weight")
+        gate, up = get(self.names["gate"]), get(self.names["up"])
         dtype = placement.common_dtype([gate, up])
         fused = torch.empty((2 * FF, H), dtype=dtype, device=placement.device)
         view = fused.view(FF // g, 2, g, H)
         view[:, 0].copy_(gate.view(FF // g, g, H))
         view[:, 1].copy_(up.view(FF // g, g, H))
         self.w_gate_up = placement.matrix(fused)
-        self.w_down = placement.place_matrix(get("down_proj.weight"))
+        self.w_down = placement.place_matrix(get(self.names["down"]))
 
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): one kernel applies the norm, both projections and the activation.
         rms = norm.fused_rms()
-        return (rms is not None and self.group == 16 and step.act_dtype == torch.bfloat16
+        return (rms is not None and self.group == 16 and self.activation == "silu" and step.act_dtype == torch.bfloat16
                 and ops.gemv_norm_supported(h, rms[0], self.w_gate_up, h.shape[0], gated=True, choices=step.choices))
 
     def forward(self, x, step, out, accumulate, pre_norm=None):
@@ -54,8 +60,13 @@ class GatedMLP(FeedForward):
             ops.gemv_norm(x, weight, eps, self.w_gate_up, act, gated=True)
         else:
             act = step.buffer("mlp.act", (T, FF), x.dtype)
-            ops.gemm_gated(x, self.w_gate_up, act, self.group,
-                           lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype), choices=step.choices)
+            if self.activation == "silu":
+                ops.gemm_gated(x, self.w_gate_up, act, self.group,
+                               lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype), choices=step.choices)
+            else:
+                gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
+                ops.gemm(x, self.w_gate_up, gu, choices=step.choices)
+                ops.gated_activation(gu, act, self.group, self.activation)
         ops.gemm(act, self.w_down, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
 
 

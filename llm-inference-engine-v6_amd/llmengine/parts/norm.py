@@ -13,16 +13,17 @@ from .registry import register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
         self.size = int(size)
         self.eps = float(eps)
+        self.tensor = tensor            # the local name of the weight ("": the part's own name)
         self.weight: torch.Tensor | None = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.size,), "norm")}
+        return {self.tensor: ParamSpec((self.size,), "norm")}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
-        self.weight = placement.place(get("weight"))
+        self.weight = placement.place(get(self.tensor))
 
     def forward(self, x, out, rows=None):
         ops.rmsnorm(x, self.weight, self.eps, out, rows)

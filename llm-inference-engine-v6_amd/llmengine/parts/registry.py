@@ -42,9 +42,9 @@ class LayerSpec:
     their sizes. `position` is handed to the mixer as its position encoding."""
     block: PartChoice
     mixer: PartChoice
-    feed_forward: PartChoice
+    feed_forward: PartChoice | None         # None: the layer is its mixer alone
     mixer_norm: PartChoice
-    ffn_norm: PartChoice
+    ffn_norm: PartChoice | None
     position: PartChoice | None = None
 
 
@@ -66,7 +66,8 @@ def build_layer(spec: LayerSpec, shared_positions: dict | None = None):
     return make_part(
         "block", spec.block.name,
         mixer=make_part("mixer", spec.mixer.name, **mixer_args),
-        feed_forward=make_part("feed_forward", spec.feed_forward.name, **spec.feed_forward.args),
+        feed_forward=(make_part("feed_forward", spec.feed_forward.name, **spec.feed_forward.args)
+                      if spec.feed_forward is not None else None),
         mixer_norm=make_part("norm", spec.mixer_norm.name, **spec.mixer_norm.args),
-        ffn_norm=make_part("norm", spec.ffn_norm.name, **spec.ffn_norm.args),
+        ffn_norm=make_part("norm", spec.ffn_norm.name, **spec.ffn_norm.args) if spec.ffn_norm is not None else None,
         **spec.block.args)

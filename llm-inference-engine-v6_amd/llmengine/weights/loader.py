@@ -24,7 +24,13 @@ class WeightError(RuntimeError):
 
 
 def _fmt(shape) -> str:
-    return "[" + ",".join(str(int(d)) for d in shape) + "]"
+    return "[" + ",".join("*" if d is None else str(int(d)) for d in shape) + "]"
+
+
+def _fits(have, want) -> bool:
+    """A stored shape against an expected one, whose None entries take any size."""
+    have, want = tuple(have), tuple(want)
+    return len(have) == len(want) and all(w is None or int(h) == int(w) for h, w in zip(have, want))
 
 
 def check_names(model: Part, available: dict[str, tuple[int, ...]], where: str, dtypes: dict | None = None) -> None:
@@ -37,7 +43,7 @@ def check_names(model: Part, available: dict[str, tuple[int, ...]], where: str, 
     missing = sorted(n for n in expected if n not in available)
     unexpected = sorted(n for n in available if n not in expected and n not in ignored and n not in aliases)
     wrong = sorted((n, expected[n].shape, available[n]) for n in expected
-                   if n in available and tuple(available[n]) != tuple(expected[n].shape))
+                   if n in available and not _fits(available[n], expected[n].shape))
     disagree = sorted((a, t) for a, t in aliases.items() if a in available and t in available and (
         tuple(available[a]) != tuple(available[t]) or (dtypes is not None and dtypes.get(a) != dtypes.get(t))))
     if not (missing or unexpected or wrong or disagree):

@@ -28,9 +28,16 @@ def _tensor_seed(seed: int, name: str) -> int:
 
 def random_tensor(name: str, shape: tuple[int, ...], init: str, seed: int, dtype: torch.dtype,
                   std: float, norm_mean: float, norm_std: float) -> torch.Tensor:
+    if any(d is None for d in shape):
+        raise ValueError(f"random weights: the shape of {name} ({shape}) has a size that only a checkpoint gives; "
+                         "name it in the configuration")
     gen = torch.Generator(device="cpu")
     gen.manual_seed(_tensor_seed(seed, name))
-    if init == "norm":
+    if init == "identity":
+        t = torch.randn(shape, generator=gen, dtype=torch.float32) * std + torch.eye(shape[-2], shape[-1])
+    elif init == "taps":
+        t = torch.randn(shape, generator=gen, dtype=torch.float32) * 0.5
+    elif init == "norm":
         if norm_std == 0.0:
             t = torch.full(shape, float(norm_mean), dtype=torch.float32)
         else:
