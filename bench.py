@@ -16,6 +16,9 @@ run at the configured context length. One JSON line goes to stdout.
 `--shape 3b` and `--shape 8b` take the layer sizes of Llama 3.2 3B and Llama 3.1 8B instead (for
 measurements at further sizes and context lengths; the default run is the 1B shape).
 
+`--phase design` runs the Rilonex design (recurrent, delta-rule and softmax-free attention layers around
+a residual in several streams) beside Llama with layers of the same sizes: prefill and decode of both.
+
 `--phase mixed` times one step of continuous batching (a prompt portion beside decoded tokens of
 other requests), `--phase portion` portions of one long prompt. `--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
 tokens and 128 to 512 new tokens each, 2,048 prompt tokens a step at most) through the
@@ -60,6 +63,94 @@ SHAPES = {
                num_key_value_heads=8, head_dim=128, tie_word_embeddings=False,
                rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0)),
 }
+
+
+# --phase design: the Rilonex design beside Llama at equal size. A size is (width, feed-forward, heads of 64);
+# Rilonex layers go rglru, channel_delta, parallel in turn, with mixers sized to a Llama layer's attention.
+DESIGN_SIZES = {"1k": (1024, 4096, 16), "2k": (2048, 8192, 32), "4k": (4096, 14336, 64)}
+
+
+def llama_at(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
+    return dict(LLAMA_1B, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), head_dim=64, vocab_size=vocab, tie_word_embeddings=False)
+
+
+def rilonex_at(width: int, ff: int, heads: int, layers: int, vocab: int, streams: int = 4, only: str = "") -> dict:
+    mlp = {"kind": "dense", "ff": ff}
+    kinds = {
+        "rglru": {"type": "rglru", "mixer": {"width": width, "blocks": max(1, width // 128), "conv": 4}, "mlp": mlp},
+        "channel_delta": {"type": "channel_delta",
+                          "mixer": {"heads": heads // 2, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4,
+                                    "decay_rank": 64, "gate_rank": 64}, "mlp": mlp},
+        "parallel": {"type": "parallel",
+                     "mixer": {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125,
+                                        "rot": {"dims": 64, "base": 10000.0}},
+                               "right": {"heads": heads // 2, "kv_heads": heads // 2, "dim": 64, "vdim": 64, "conv": 4},
+                               "left_scale": 0.5, "right_scale": 0.5}, "mlp": mlp},
+    }
+    order = [only] if only else ["rglru", "channel_delta", "parallel"]
+    return {"architecture": "Rilonex", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": 1e-5},
+            "layers": [kinds[order[i % len(order)]] for i in range(layers)]}
+
+
+def design(args) -> int:
+    """Prefill (one prompt of --prefill-tokens) and decode (--batch requests at --context) of the Rilonex design and of
+    Llama with layers of the same width, feed-forward size and number of heads: tokens/s of both and their ratio, per
+    size of DESIGN_SIZES named in --design-sizes; --design-only times a Rilonex of one kind of layer."""
+    import torch
+    from llmengine import Engine, StepEntry
+    layers = args.layers or 6
+    vocab, page, T = 32768, args.page_size, args.prefill_tokens
+    rows = []
+    for size in [x for x in args.design_sizes.split(",") if x]:
+        width, ff, heads = DESIGN_SIZES[size]
+        row = {"size": size, "width": width, "ff": ff, "heads": heads, "layers": layers}
+        for name, cfg in (("llama", llama_at(width, ff, heads, layers, vocab)),
+                          ("rilonex", rilonex_at(width, ff, heads, layers, vocab, only=args.design_only))):
+            engine = Engine.from_random(cfg, args.seed, args.dtype, std=0.02)
+            gen = torch.Generator().manual_seed(args.seed + 1)
+            prompt = torch.randint(0, vocab, (T,), generator=gen).tolist()
+            cache = engine.new_cache((T + page - 1) // page + 1, page, 1)
+            times = []
+            for rep in range(5):
+                cache.admit("p")
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                engine.step(cache, [StepEntry("p", prompt, [T - 1])])
+                torch.cuda.synchronize()
+                times.append((time.perf_counter() - t) * 1e3)
+                cache.release("p")
+            pre_ms = min(times[1:])
+            del cache
+            batch, steps, warm = args.batch, max(16, min(args.steps, 64)), 4
+            start = args.context - steps - warm
+            cache = engine.new_cache(batch * ((args.context + page - 1) // page + 1), page, batch)
+            ids = list(range(batch))
+            for rid in ids:
+                cache.admit(rid)
+                toks = torch.randint(0, vocab, (start,), generator=gen).tolist()
+                for s in range(0, start, 2048):
+                    engine.step(cache, [StepEntry(rid, toks[s:s + 2048], [])])
+            last = engine.greedy_chain(cache, ids, [1] * batch, warm)[-1]
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.greedy_chain(cache, ids, last, steps)
+            torch.cuda.synchronize()
+            dec_ms = (time.perf_counter() - t) / steps * 1e3
+            row[name] = {"prefill_ms": round(pre_ms, 3), "prefill_tok_s": round(T / pre_ms * 1e3, 1),
+                         "decode_ms": round(dec_ms, 4), "decode_tok_s": round(batch / dec_ms * 1e3, 1)}
+            log(f"{size} {name}: prefill {T} tokens {pre_ms:.2f} ms, decode b{batch} ctx {args.context} {dec_ms:.3f} ms/step")
+            del cache, engine
+            torch.cuda.empty_cache()
+        row["prefill_ratio"] = round(row["rilonex"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["rilonex"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3)
+        rows.append(row)
+    print(json.dumps({"metric": "design_tokens_per_second_beside_llama", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
+                      "value": rows[0]["rilonex"]["decode_tok_s"] if rows else None,
+                      "config": {"prefill_tokens": T, "batch": args.batch, "context": args.context, "page_size": page,
+                                 "vocab": vocab, "only": args.design_only or "rglru, channel_delta, parallel in turn"},
+                      "sizes": rows}), flush=True)
+    return 0
 
 
 def log(msg: str) -> None:
@@ -248,11 +339,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve", "portion", "mixed"],
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve", "portion", "mixed", "design"],
                     help="run only one part (for profiling); the JSON line then lacks the other. 'serve' is another "
                          "workload: requests of mixed lengths through the continuous-batching scheduler; 'portion': "
                          "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
                          "portion beside one decoded token of --batch other requests")
+    ap.add_argument("--design-sizes", default="1k,2k", help="design: sizes to run, of " + ",".join(sorted(DESIGN_SIZES)))
+    ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel"],
+                    help="design: a Rilonex of this kind of layer only")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--decode-len", type=int, default=700, help="mixed: tokens of the shortest decoding request "
                                                                 "(the longest has 800 more)")
@@ -268,6 +362,9 @@ def main() -> int:
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.phase == "design":
+        return design(args)
 
     import torch
     from llmengine import Engine, StepEntry

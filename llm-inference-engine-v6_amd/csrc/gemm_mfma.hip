@@ -51,7 +51,14 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 // The fourth word of a buffer descriptor for raw 32-bit data on this chip.
 constexpr int kBufferFlags = 0x00020000;
 
-enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4, kRopeCache = 5 };
+enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4, kRopeCache = 5,
+                     kGatedReluBF16 = 6 };
+// The gated outputs: act(gate) * up with act = SiLU (kGatedBF16) or the rectifier (kGatedReluBF16).
+constexpr bool is_gated(int mode) { return mode == kGatedBF16 || mode == kGatedReluBF16; }
+template <int MODE> __device__ __forceinline__ float gate_act(float g) {
+    if (MODE == kGatedReluBF16) return fmaxf(g, 0.f);
+    return g / (1.0f + expf(-g));
+}
 
 // Where the q/k/v projection's epilogue (kRopeCache) puts its result: the columns are the heads
 // of q, then k, then v (hd columns each); q and k heads are rotated at the rows' positions (pairs
@@ -235,7 +242,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                     }
                 }
             }
-        } else if (MODE == kGatedBF16) {
+        } else if (is_gated(MODE)) {
             // a thread makes 8 units: their gates and ups lie 16 columns apart in a group of 32
             constexpr int PER_ROW = BN / 16;             // 8-unit pieces per row
             for (int idx = tid; idx < HB * PER_ROW; idx += NT) {
@@ -248,7 +255,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float gt = gp[e], up = gp[16 + e];
-                    o[e] = static_cast<__bf16>((gt / (1.0f + expf(-gt))) * up);
+                    o[e] = static_cast<__bf16>(gate_act<MODE>(gt) * up);
                 }
                 const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
                 *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * (N / 2) + unit) = o;
@@ -307,14 +314,14 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
         for (int e = 0; e < 4; ++e) {
             const int m = m0 + wm + i * 16 + q * 4 + e;
             if (m >= M) continue;
-            if (MODE == kGatedBF16) {
+            if (is_gated(MODE)) {
 #pragma unroll
                 for (int j = 0; j + 1 < WNT; j += 2) {
                     const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
                     if (2 * unit >= N) continue;
                     const float gt = acc[i][j][e], up = acc[i][j + 1][e];
                     static_cast<bf16*>(out)[static_cast<size_t>(m) * (N / 2) + unit] =
-                        static_cast<bf16>((gt / (1.0f + expf(-gt))) * up);
+                        static_cast<bf16>(gate_act<MODE>(gt) * up);
                 }
             } else {
 #pragma unroll
@@ -774,6 +781,7 @@ static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, in
         case kAddF32: return launch_tile_mode<WMT, WNT, kAddF32>(A, W, out, M, N, K, 1, blocked, stream);
         case kAtomicF32: return launch_tile_mode<WMT, WNT, kAtomicF32>(A, W, out, M, N, K, ksplit, blocked, stream);
         case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, blocked, stream);
+        case kGatedReluBF16: return launch_tile_mode<WMT, WNT, kGatedReluBF16>(A, W, out, M, N, K, 1, blocked, stream);
         default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, blocked, stream);
     }
 }
@@ -791,6 +799,7 @@ static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, in
         case kAddF32: return LLME_DIRECT(kAddF32);
         case kAtomicF32: return LLME_DIRECT(kAtomicF32);
         case kGatedBF16: return LLME_DIRECT(kGatedBF16);
+        case kGatedReluBF16: return LLME_DIRECT(kGatedReluBF16);
         default: return LLME_DIRECT(kStoreBF16);
     }
 #undef LLME_DIRECT
@@ -982,7 +991,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // tile shape: 0 lets the entry point choose: the largest tile that still gives about one
     // workgroup per compute unit; a small output with a long k is cut over k instead (the
     // parts are added with atomics, so this needs an accumulating float32 output).
-    if (gated) mode = kGatedBF16;
+    if (gated) mode = gated == 2 ? kGatedReluBF16 : kGatedBF16;
     const bool auto_shape = tile_shape <= 0;
     float tiles_cost = -1.f;                           // of the chosen tile, in the units of the estimate below
     if (tile_shape <= 0) {
@@ -1013,7 +1022,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
                 float cost = static_cast<float>(rounds) * heights[c] * widths[c] / eff[c];
                 // (less so for the gated product, whose epilogue is long: measured at 129 to 256 rows,
                 // 128 x 128 tiles 26.5 against 31 us at the 1B sizes, 36.6 against 43.7 at the 3B sizes)
-                if (wgs <= cus) cost *= (mode == kGatedBF16 ? 1.1f : 1.25f);
+                if (wgs <= cus) cost *= (is_gated(mode) ? 1.1f : 1.25f);
                 if (c == 0 || cost < best) {
                     best = cost;
                     tile_shape = shapes[c];

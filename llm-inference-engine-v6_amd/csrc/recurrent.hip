@@ -158,6 +158,67 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(const float* __restrict
     *st = h;
 }
 
+// The same recurrence for long runs of rows, in three passes over chunks of `chunk` rows of a request:
+// (1) every chunk's product of decays P and its result from an empty state B; (2) per request and channel, the state in
+// front of every chunk (carry_j+1 = P_j carry_j + B_j, from the slot's state, which becomes the last one); (3) every
+// chunk again from its carry, with the outputs. part [n_seq, chunks, 2, width] holds (P, B), then (carry, -).
+__global__ __launch_bounds__(256) void rglru_chunk_sums_kernel(const float* __restrict__ decay, const float* __restrict__ drive,
+                                                               const int* __restrict__ q_start, float* __restrict__ part,
+                                                               int width, int chunk, int chunks) {
+    const int s = blockIdx.z, j = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int first = q_start[s] + j * chunk;
+    const int last = min(q_start[s + 1], first + chunk);
+    if (c >= width || first >= last) return;
+    float p = 1.f, h = 0.f;
+    for (int t = first; t < last; ++t) {
+        const size_t at = static_cast<size_t>(t) * width + c;
+        const float a = decay[at];
+        p *= a;
+        h = a * h + drive[at];
+    }
+    float* out = part + (static_cast<size_t>(s) * chunks + j) * 2 * width;
+    out[c] = p;
+    out[width + c] = h;
+}
+
+__global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(float* __restrict__ part, float* __restrict__ state,
+                                                                const int* __restrict__ q_start, const int* __restrict__ slots,
+                                                                int width, int chunk, int chunks) {
+    const int s = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= width) return;
+    const int n = q_start[s + 1] - q_start[s];
+    float* st = state + static_cast<size_t>(slots[s]) * width + c;
+    float h = *st;
+    for (int j = 0; j * chunk < n; ++j) {
+        float* pb = part + (static_cast<size_t>(s) * chunks + j) * 2 * width;
+        const float p = pb[c], b = pb[width + c];
+        pb[c] = h;
+        h = p * h + b;
+    }
+    *st = h;
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void rglru_chunk_scan_kernel(const float* __restrict__ decay, const float* __restrict__ drive,
+                                                               const float* __restrict__ y, int ld_y, const float* __restrict__ yb,
+                                                               const float* __restrict__ part, const int* __restrict__ q_start,
+                                                               TO* __restrict__ out, int ld_out, int width, int chunk, int chunks) {
+    const int s = blockIdx.z, j = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int first = q_start[s] + j * chunk;
+    const int last = min(q_start[s + 1], first + chunk);
+    if (c >= width || first >= last) return;
+    float h = part[(static_cast<size_t>(s) * chunks + j) * 2 * width + c];
+    const float bias = yb ? yb[c] : 0.f;
+    for (int t = first; t < last; ++t) {
+        const size_t at = static_cast<size_t>(t) * width + c;
+        h = decay[at] * h + drive[at];
+        out[static_cast<size_t>(t) * ld_out + c] = from_float<TO>(h * gelu_tanhf_(y[static_cast<size_t>(t) * ld_y + c] + bias));
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // x <- x / sqrt(sum(x^2) + eps) * scale over every head of `dim` entries, in place; heads [0, n_a) scale by
 // scale_a, heads [n_a, n_a + n_b) by scale_b (queries and keys lie side by side). One wavefront per (row, head).
@@ -359,6 +420,35 @@ extern "C" int llme_rglru_scan(const void* decay, const void* drive, const void*
         default: return kErrBadArgument;
     }
 #undef LLME_SCAN
+    return launch_status();
+}
+
+// The chunked form: part is scratch of n_seq * chunks * 2 * width floats, chunks >= ceil(longest request's rows / chunk).
+extern "C" int llme_rglru_scan_chunked(const void* decay, const void* drive, const void* y, int ld_y, const void* yb,
+                                       void* state, const void* q_start, const void* slots, void* out, int out_dtype,
+                                       int ld_out, int n_seq, int width, int chunk, int chunks, void* part,
+                                       hipStream_t stream) {
+    if (n_seq <= 0 || width <= 0) return 0;
+    if (chunk <= 0 || chunks <= 0) return kErrBadArgument;
+    const dim3 grid((width + 255) / 256, chunks, n_seq);
+    const float* dp = static_cast<const float*>(decay);
+    const float* vp = static_cast<const float*>(drive);
+    const int* qs = static_cast<const int*>(q_start);
+    float* pp = static_cast<float*>(part);
+    rglru_chunk_sums_kernel<<<grid, 256, 0, stream>>>(dp, vp, qs, pp, width, chunk, chunks);
+    rglru_chunk_carry_kernel<<<dim3((width + 255) / 256, n_seq), 256, 0, stream>>>(pp, static_cast<float*>(state), qs,
+                                                                                   static_cast<const int*>(slots), width, chunk,
+                                                                                   chunks);
+    if (out_dtype == kF32)
+        rglru_chunk_scan_kernel<float><<<grid, 256, 0, stream>>>(dp, vp, static_cast<const float*>(y), ld_y,
+                                                                 static_cast<const float*>(yb), pp, qs,
+                                                                 static_cast<float*>(out), ld_out, width, chunk, chunks);
+    else if (out_dtype == kBF16)
+        rglru_chunk_scan_kernel<bf16><<<grid, 256, 0, stream>>>(dp, vp, static_cast<const float*>(y), ld_y,
+                                                                static_cast<const float*>(yb), pp, qs, static_cast<bf16*>(out),
+                                                                ld_out, width, chunk, chunks);
+    else
+        return kErrBadArgument;
     return launch_status();
 }
 

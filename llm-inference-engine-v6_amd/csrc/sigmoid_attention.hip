@@ -19,7 +19,8 @@ namespace llme {
 
 // q, k heads of qkvg [T, ld] (32-bit; q at column 0, k behind the q heads, v behind the k heads): entry i < rot / 2
 // of a head turns with entry i + rot / 2 by the angle position * inv_freq[i] (a 32-bit product); q goes to q_out
-// [T, H * dim], k and v into the row's page: k_cache [pages, G, page, dim], v_cache [pages, G, page, vdim].
+// [T, H * dim], k and v into the row's page: k_cache [pages, G, page, dim], v_cache [pages, G, vdim, page] (a value
+// channel's tokens lie together, as the matrix instructions of the second product read them).
 template <typename TQ, typename TC>
 __global__ __launch_bounds__(256) void rotate_write_kernel(const float* __restrict__ qkv, int ld, const float* __restrict__ inv_freq,
                                                            const int* __restrict__ positions, const int* __restrict__ seq_idx,
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(256) void rotate_write_kernel(const float* __restri
     const float* vp = row + static_cast<size_t>(H + G) * dim;
     for (int e = threadIdx.x; e < G * vdim; e += 256) {
         const int head = e / vdim, i = e % vdim;
-        v_cache[((static_cast<size_t>(pg) * G + head) * page + in_page) * vdim + i] = from_float<TC>(vp[e]);
+        v_cache[((static_cast<size_t>(pg) * G + head) * vdim + i) * page + in_page] = from_float<TC>(vp[e]);
     }
 }
 
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_kernel(const TQ* __rest
                     float a = acc[i];
                     for (int j = 0; j < nk; ++j) {
                         const int key = j0 + j;
-                        a += wp[j] * to_float(v_cache[((static_cast<size_t>(table[key / page]) * G + h / per) * page + key % page) * vdim + x]);
+                        a += wp[j] * to_float(v_cache[((static_cast<size_t>(table[key / page]) * G + h / per) * vdim + x) * page + key % page]);
                     }
                     acc[i] = a;
                 }
@@ -136,6 +137,181 @@ __global__ __launch_bounds__(256) void sigmoid_attention_kernel(const TQ* __rest
         const int e = tid + 256 * i;
         if (e < H * vdim) out[e] = acc[i];
     }
+}
+
+// The same on the matrix cores, for bfloat16 rows that come at least 16 to a request (prompts and their portions).
+// A workgroup owns 16 consecutive rows of one request and one run of its keys; each of its H / 4 wavefronts owns four
+// heads. Per tile of 32 keys: (1) every wavefront makes the transposed scores K Q^T of its heads (so that a lane holds,
+// for one query, the keys that the second product wants from it) and puts them, scaled, into LDS; (2) it mixes all
+// heads' scores into its own heads' (32-bit FMAs against the mixing matrix, broadcast from LDS), makes the weights,
+// splits each into two bfloat16 parts (w = hi + lo, 16 bits of mantissa) and adds both parts' products with V.
+// Weights of keys behind a row's position are zero. Partial sums go where the finishing kernel adds the runs.
+typedef __attribute__((ext_vector_type(8))) __bf16 sa_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 sa_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float sa_f32x4;
+
+template <int DIM32, int VT>
+__global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const float* __restrict__ mix_t, const float* __restrict__ bias, const int* __restrict__ positions,
+    const int* __restrict__ q_start, const int* __restrict__ block_table, int max_blocks, float* __restrict__ partial,
+    int T, int n_seq, int H, int G, int page, float scale, int run_len) {
+    constexpr int DIM = DIM32 * 32, VDIM = VT * 16, HPW = 4;
+    extern __shared__ float lds[];
+    float* sc = lds;                        // [H][64 lanes][8]
+    float* mt = sc + H * 512;               // [H (from)][H (to)]
+    float* bs = mt + H * H;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int r16 = lane % 16, q4 = lane / 16;
+    // which request and which 16 of its rows
+    int item = blockIdx.x, s = 0, row0 = 0, nrows = 0;
+    for (; s < n_seq; ++s) {
+        const int n = q_start[s + 1] - q_start[s];
+        const int tiles = (n + 15) / 16;
+        if (item < tiles) {
+            row0 = q_start[s] + item * 16;
+            nrows = min(16, q_start[s + 1] - row0);
+            break;
+        }
+        item -= tiles;
+    }
+    if (s >= n_seq) return;
+    const int run = blockIdx.y;
+    const int* table = block_table + static_cast<size_t>(s) * max_blocks;
+    const int my_row = row0 + min(r16, nrows - 1);
+    const int my_pos = positions[my_row];
+    const int kmax = positions[row0 + nrows - 1];
+    const int key_lo = run * run_len, key_hi = min(kmax + 1, key_lo + run_len);
+    for (int e = threadIdx.x; e < H * H; e += blockDim.x) mt[e] = mix_t[e];
+    for (int e = threadIdx.x; e < H; e += blockDim.x) bs[e] = bias[e];
+    const int h0 = wave * HPW, per = H / G;
+    sa_bf16x8 qf[HPW][DIM32];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+        for (int c = 0; c < DIM32; ++c)
+            qf[hh][c] = *reinterpret_cast<const sa_bf16x8*>(q + (static_cast<size_t>(my_row) * H + h0 + hh) * DIM + c * 32 + q4 * 8);
+    sa_f32x4 o[HPW][VT];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+        for (int dt = 0; dt < VT; ++dt) o[hh][dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    for (int j0 = key_lo; j0 < key_hi; j0 += 32) {
+        // (1) transposed scores of this wavefront's heads
+        {
+            int have = -1;
+            sa_bf16x8 kf[2][DIM32];
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int g = h0 + hh, kv = g / per;
+                if (kv != have) {
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt) {
+                        const int key = min(j0 + rt * 16 + r16, kmax);
+                        const bf16* kp = k_cache + ((static_cast<size_t>(table[key / page]) * G + kv) * page + key % page) * DIM;
+#pragma unroll
+                        for (int c = 0; c < DIM32; ++c) kf[rt][c] = *reinterpret_cast<const sa_bf16x8*>(kp + c * 32 + q4 * 8);
+                    }
+                    have = kv;
+                }
+                sa_f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < DIM32; ++c) {
+                    a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][c], qf[hh][c], a0, 0, 0, 0);
+                    a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][c], qf[hh][c], a1, 0, 0, 0);
+                }
+                float* dst = sc + (static_cast<size_t>(g) * 64 + lane) * 8;
+                *reinterpret_cast<float4*>(dst) = float4{a0[0] * scale, a0[1] * scale, a0[2] * scale, a0[3] * scale};
+                *reinterpret_cast<float4*>(dst + 4) = float4{a1[0] * scale, a1[1] * scale, a1[2] * scale, a1[3] * scale};
+            }
+        }
+        __syncthreads();
+        // (2) all heads' scores mixed into this wavefront's heads
+        float m[HPW][8];
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) m[hh][e] = 0.f;
+        for (int g = 0; g < H; ++g) {
+            const float4 s0 = *reinterpret_cast<const float4*>(sc + (static_cast<size_t>(g) * 64 + lane) * 8);
+            const float4 s1 = *reinterpret_cast<const float4*>(sc + (static_cast<size_t>(g) * 64 + lane) * 8 + 4);
+            const float4 tw = *reinterpret_cast<const float4*>(mt + g * H + h0);
+            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const float tv[4] = {tw.x, tw.y, tw.z, tw.w};
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) m[hh][e] += tv[hh] * sv[e];
+        }
+        {
+            int have = -1;
+            sa_bf16x8 vf[VT];
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = h0 + hh, kv = h / per;
+                const float b = bs[h];
+                sa_bf16x8 hi, lo;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int key = j0 + (e < 4 ? 4 * q4 + e : 16 + 4 * q4 + (e - 4));
+                    const float w = (key <= my_pos && key < key_hi) ? 1.0f / (1.0f + expf(-(m[hh][e] + b))) : 0.f;
+                    hi[e] = static_cast<__bf16>(w);
+                    lo[e] = static_cast<__bf16>(w - static_cast<float>(hi[e]));
+                }
+                if (kv != have) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const int key = min(j0 + half * 16 + 4 * q4, kmax & ~3);
+                        const bf16* vp = v_cache + (static_cast<size_t>(table[key / page]) * G + kv) * VDIM * page + key % page;
+#pragma unroll
+                        for (int dt = 0; dt < VT; ++dt) {
+                            const sa_bf16x4 v4 = *reinterpret_cast<const sa_bf16x4*>(vp + static_cast<size_t>(dt * 16 + r16) * page);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) vf[dt][half * 4 + e] = v4[e];
+                        }
+                    }
+                    have = kv;
+                }
+#pragma unroll
+                for (int dt = 0; dt < VT; ++dt) {
+                    o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf[dt], o[hh][dt], 0, 0, 0);
+                    o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, vf[dt], o[hh][dt], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh)
+#pragma unroll
+        for (int dt = 0; dt < VT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * q4 + r;
+                if (i < nrows)
+                    partial[((static_cast<size_t>(run) * T) + row0 + i) * H * VDIM + (h0 + hh) * VDIM + dt * 16 + r16] = o[hh][dt][r];
+            }
+}
+
+template <int DIM32, int VT>
+static int launch_sigmoid_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const float* mix_t,
+                                         const float* bias, const int* positions, const int* q_start, const int* block_table,
+                                         int max_blocks, float* partial, int T, int n_seq, int H, int G, int page, float scale,
+                                         int run_len, int runs, int tiles, hipStream_t stream) {
+    const size_t lds = sizeof(float) * (static_cast<size_t>(H) * 512 + static_cast<size_t>(H) * H + H);
+    auto kernel = sigmoid_attention_mfma_kernel<DIM32, VT>;
+    static size_t allowed = 0;
+    if (lds > 64 * 1024 && lds > allowed) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 static_cast<int>(lds));
+        if (e != hipSuccess) return static_cast<int>(e);
+        allowed = lds;
+    }
+    kernel<<<dim3(tiles, runs), (H / 4) * 64, lds, stream>>>(
+        static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), mix_t, bias, positions,
+        q_start, block_table, max_blocks, partial, T, n_seq, H, G, page, scale, run_len);
+    return launch_status();
 }
 
 // out[t, h, :] = scale_out * sigmoid(gate[t, h]) * sum_runs partial[run, t, h, :]
@@ -221,6 +397,39 @@ extern "C" int llme_sigmoid_attention(const void* q, int q_dtype, const void* k_
         case 3: return launch_sigmoid_attention<bf16, bf16>(q, k_cache, v_cache, mp, bp, pp, sp, tp, max_blocks, part, T, H, G,
                                                             dim, vdim, page, scale, run_len, runs, stream);
     }
+    return kErrUnsupported;
+}
+
+// The matrix-core form: bfloat16 q and pages, H a multiple of 4 up to 32, dim a multiple of 32 up to 128, vdim a multiple
+// of 16 up to 128, pages of a multiple of 16 tokens, run_len a multiple of 32. mix_t is the mixing matrix transposed
+// ([from, to]). tiles = sum over the requests of ceil(rows / 16).
+extern "C" int llme_sigmoid_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const void* mix_t,
+                                           const void* bias, const void* positions, const void* q_start,
+                                           const void* block_table, int max_blocks, void* partial, int T, int n_seq, int H,
+                                           int G, int dim, int vdim, int page, float scale, int run_len, int runs, int tiles,
+                                           hipStream_t stream) {
+    if (T <= 0 || tiles <= 0) return 0;
+    if (G <= 0 || H % G || runs <= 0 || run_len <= 0 || run_len % 32) return kErrBadArgument;
+    if (H % 4 || H > 32 || dim % 32 || dim > 128 || vdim % 16 || vdim > 128 || page % 16) return kErrUnsupported;
+#define LLME_SAM(D_, V_)                                                                                                 \
+    return launch_sigmoid_attention_mfma<D_, V_>(q, k_cache, v_cache, static_cast<const float*>(mix_t),                  \
+                                                 static_cast<const float*>(bias), static_cast<const int*>(positions),   \
+                                                 static_cast<const int*>(q_start), static_cast<const int*>(block_table), \
+                                                 max_blocks, static_cast<float*>(partial), T, n_seq, H, G, page, scale,  \
+                                                 run_len, runs, tiles, stream)
+#define LLME_SAM_V(D_)                                                                                                   \
+    switch (vdim / 16) {                                                                                                 \
+        case 1: LLME_SAM(D_, 1); case 2: LLME_SAM(D_, 2); case 3: LLME_SAM(D_, 3); case 4: LLME_SAM(D_, 4);              \
+        case 5: LLME_SAM(D_, 5); case 6: LLME_SAM(D_, 6); case 7: LLME_SAM(D_, 7); case 8: LLME_SAM(D_, 8);              \
+    }
+    switch (dim / 32) {
+        case 1: LLME_SAM_V(1) break;
+        case 2: LLME_SAM_V(2) break;
+        case 3: LLME_SAM_V(3) break;
+        case 4: LLME_SAM_V(4) break;
+    }
+#undef LLME_SAM_V
+#undef LLME_SAM
     return kErrUnsupported;
 }
 

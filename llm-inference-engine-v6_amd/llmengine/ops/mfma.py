@@ -25,11 +25,11 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, acc
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, *,
-              gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False,
+              gated: bool | str = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False,
               direct: int = -1, _supported: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
     K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
-    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064, 96128, 96064) /
+    out is bfloat16 [M, N / 2] = silu(gate) * up (gated="relu": the rectifier instead of SiLU). waves / ksplit / tile (64, 128, 128096, 128064, 96128, 96064) /
     force_tile override the launch choices (tests and measurements); direct: whether the product may
     use the 256 x 256 tile kernel whose slabs go from memory straight into LDS, which needs a blocked w
     (-1: where it pays, 0: never, 1: it must, with tile 256256)."""
@@ -48,30 +48,36 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     if force_tile and not tile:
         tile = 128
     check(entry("llme_gemm_bf16")(ptr(a), ptr(w), ptr(out), 0 if out.dtype == torch.float32 else 1, M, N, K,
-                                  1 if accumulate else 0, 1 if gated else 0, waves, ksplit, tile,
+                                  1 if accumulate else 0, (2 if gated == "relu" else 1) if gated else 0, waves, ksplit, tile,
                                   1 if kernels.is_blocked(w) else 0, int(direct), stream()),
           "gemm_bf16")
 
 
 def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, group: int, scratch,
-               choices: KernelChoices | None = None) -> None:
-    """out [T, FF] = silu(x Wg^T) * (x Wu^T), the gate and up rows interleaved in groups of `group`
+               choices: KernelChoices | None = None, activation: str = "silu") -> None:
+    """out [T, FF] = act(x Wg^T) * (x Wu^T) (act SiLU unless named otherwise), the gate and up rows interleaved in groups of `group`
     rows of w_gate_up [2 FF, K]. One MFMA kernel where the types and sizes fit it; otherwise the
     product into a 32-bit scratch [T, 2 FF] (scratch(shape, dtype) provides it) and the
     activation kernel."""
     T, FF = out.shape
     if ((choices or DEFAULT).fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
+            and activation in ("silu", "relu")
             and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
         r = tail_rows(T, choices)
+        mode = "relu" if activation == "relu" else True
         if r:
-            gemm_bf16(x[:T - r], w_gate_up, out[:T - r], gated=True, _supported=True)
-            gemm_bf16(x[T - r:], w_gate_up, out[T - r:], gated=True, _supported=True)
+            gemm_bf16(x[:T - r], w_gate_up, out[:T - r], gated=mode, _supported=True)
+            gemm_bf16(x[T - r:], w_gate_up, out[T - r:], gated=mode, _supported=True)
             return
-        gemm_bf16(x, w_gate_up, out, gated=True, _supported=True)
+        gemm_bf16(x, w_gate_up, out, gated=mode, _supported=True)
         return
     gu = scratch((T, 2 * FF), torch.float32)
     kernels.gemm(x, w_gate_up, gu, choices=choices)
-    kernels.swiglu(gu, out, group)
+    if activation == "silu":
+        kernels.swiglu(gu, out, group)
+    else:
+        from .recurrent import gated_activation
+        gated_activation(gu, out, group, activation)
 
 
 declare("llme_gemm_bf16_qkv_rope", [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])

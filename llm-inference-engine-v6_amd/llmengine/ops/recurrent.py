@@ -19,6 +19,7 @@ _FLOATS = (torch.float32, torch.bfloat16)
 MAX_STREAMS = 8
 MAX_TAPS = 16
 DELTA_MAX_DIM = 256
+RGLRU_CHUNK_FROM, RGLRU_CHUNK = 64, 32        # requests that bring more rows than the first are scanned in chunks of the second
 GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
 
 declare("llme_streams_spread", [_vp, _i, _z, _vp])
@@ -28,12 +29,14 @@ declare("llme_gated_act", [_vp, _i, _vp, _i, _i, _i, _i, _i, _vp])
 declare("llme_short_conv", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_rglru_gates", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp])
 declare("llme_rglru_scan", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
+declare("llme_rglru_scan_chunked", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp])
 declare("llme_unit_heads", [_vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp])
 declare("llme_delta_gates", [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp])
 declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
 declare("llme_gated_head_norm", [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _f, _vp])
 declare("llme_rotate_write", [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_sigmoid_attention", [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp])
+declare("llme_sigmoid_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _vp])
 declare("llme_sigmoid_attention_finish", [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _vp])
 
 
@@ -172,6 +175,16 @@ def rglru_scan(decay: torch.Tensor, drive: torch.Tensor, y: torch.Tensor, y_bias
     ld_out = _cols(out, "out", _FLOATS, T, width)
     if T != step.num_tokens:
         raise KernelError("rglru_scan: one row per token of the step")
+    longest = max(step.new_lens) if step.new_lens else T
+    if longest > RGLRU_CHUNK_FROM:
+        # long runs of rows (prompts): chunks scanned side by side, joined through each chunk's (product, sum)
+        chunk = RGLRU_CHUNK
+        chunks = (longest + chunk - 1) // chunk
+        part = step.buffer("rglru.chunks", (step.num_seqs, chunks, 2, width), torch.float32)
+        check(entry("llme_rglru_scan_chunked")(ptr(decay), ptr(drive), ptr(y), ld_y, ptr(y_bias), ptr(state), ptr(step.q_start),
+                                               ptr(step.slots), ptr(out), code(out.dtype), ld_out, step.num_seqs, width, chunk,
+                                               chunks, ptr(part), stream()), "rglru_scan_chunked")
+        return
     check(entry("llme_rglru_scan")(ptr(decay), ptr(drive), ptr(y), ld_y, ptr(y_bias), ptr(state), ptr(step.q_start),
                                    ptr(step.slots), ptr(out), code(out.dtype), ld_out, step.num_seqs, width, stream()),
           "rglru_scan")
@@ -260,7 +273,7 @@ def rotate_write(qkv: torch.Tensor, inv_freq: torch.Tensor | None, step, block_t
                  k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int) -> None:
     """Rotates the q and k heads of qkv [T, heads dim + kv_heads dim + kv_heads vdim] (32-bit) by position * inv_freq
     (pairs (i, i + r / 2), r = 2 len(inv_freq); None: no rotation), writes q to q_out [T, heads dim] and k, v into the
-    rows' pages: k_cache [pages, kv_heads, page, dim], v_cache [pages, kv_heads, page, vdim]."""
+    rows' pages: k_cache [pages, kv_heads, page, dim], v_cache [pages, kv_heads, vdim, page]."""
     T = qkv.shape[0]
     ld = _cols(qkv, "qkv", torch.float32, T, (heads + kv_heads) * dim + kv_heads * vdim)
     rot = 0
@@ -272,7 +285,7 @@ def rotate_write(qkv: torch.Tensor, inv_freq: torch.Tensor | None, step, block_t
     require(q_out, "q_out", _FLOATS, (T, heads * dim))
     require(k_cache, "k_cache", _FLOATS, (None, kv_heads, None, dim))
     page = k_cache.shape[2]
-    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], kv_heads, page, vdim))
+    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], kv_heads, vdim, page))
     require(block_table, "block_table", torch.int32, (None, None))
     check(entry("llme_rotate_write")(ptr(qkv), ld, ptr(inv_freq), ptr(step.positions), ptr(step.seq_idx), ptr(block_table),
                                      block_table.shape[1], ptr(q_out), code(q_out.dtype), ptr(k_cache), ptr(v_cache),
@@ -286,9 +299,18 @@ def sigmoid_attention_fits(heads: int, dim: int, vdim: int) -> bool:
     return 4 * (heads * dim + heads * heads + heads + 2 * heads * 32) <= SIGMOID_ATTENTION_LDS and heads * vdim <= 256 * 32
 
 
+def sigmoid_attention_mfma_fits(q: torch.Tensor, heads: int, dim: int, vdim: int, page: int) -> bool:
+    """Whether the matrix-core kernel takes these operands (bfloat16, four heads per wavefront, whole matrix tiles)."""
+    return (q.dtype == torch.bfloat16 and heads % 4 == 0 and heads <= 32 and dim % 32 == 0 and dim <= 128
+            and vdim % 16 == 0 and vdim <= 128 and page % 16 == 0)
+
+
+SIGMOID_ATTENTION_MFMA_ROWS = 16        # a request must bring this many rows for the step to take the matrix-core kernel
+
+
 def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, mix: torch.Tensor, bias: torch.Tensor,
                       gate: torch.Tensor, step, block_table: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
-                      dim: int, vdim: int, scale: float, scale_out: float = 1.0) -> None:
+                      dim: int, vdim: int, scale: float, scale_out: float = 1.0, mix_t: torch.Tensor | None = None) -> None:
     """out[t, h] = scale_out * sigmoid(gate[t, h]) * sum_(j <= pos) sigmoid(sum_g mix[h, g] s[g, j] + bias[h]) v_j with
     s[g, j] = scale q_g . k_j over the row's pages. The keys of long requests are cut into runs (one workgroup
     each) whose partial sums are added in a fixed order."""
@@ -296,7 +318,7 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     require(q, "q", _FLOATS, (T, heads * dim))
     require(k_cache, "k_cache", q.dtype, (None, kv_heads, None, dim))
     page = k_cache.shape[2]
-    require(v_cache, "v_cache", q.dtype, (k_cache.shape[0], kv_heads, page, vdim))
+    require(v_cache, "v_cache", q.dtype, (k_cache.shape[0], kv_heads, vdim, page))
     require(mix, "mix", torch.float32, (heads, heads))
     require(bias, "bias", torch.float32, (heads,))
     ld_gate = _cols(gate, "gate", torch.float32, T, heads)
@@ -310,6 +332,23 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     else:
         longest = max(c + n for c, n in zip(step.ctx_lens, step.new_lens))
     from .mfma import compute_units
+    from .choices import choices_of
+    if (step.plan_len is None and mix_t is not None and choices_of(step).fast_attention
+            and max(step.new_lens) >= SIGMOID_ATTENTION_MFMA_ROWS and sigmoid_attention_mfma_fits(q, heads, dim, vdim, page)):
+        # prompts and their portions: 16 rows of a request to a workgroup, scores and the second product on the matrix cores
+        require(mix_t, "mix_t", torch.float32, (heads, heads))
+        tiles = sum((n + 15) // 16 for n in step.new_lens)
+        runs = max(1, min(32, (2 * compute_units()) // tiles, (longest + 511) // 512))
+        run_len = ((longest + runs - 1) // runs + 31) // 32 * 32
+        runs = max(1, (longest + run_len - 1) // run_len)
+        partial = step.buffer("sigmoid_attention.partial", (runs, T, heads * vdim), torch.float32)
+        check(entry("llme_sigmoid_attention_mfma")(ptr(q), ptr(k_cache), ptr(v_cache), ptr(mix_t), ptr(bias), ptr(step.positions),
+                                                   ptr(step.q_start), ptr(block_table), block_table.shape[1], ptr(partial), T,
+                                                   step.num_seqs, heads, kv_heads, dim, vdim, page, float(scale), run_len, runs,
+                                                   tiles, stream()), "sigmoid_attention_mfma")
+        check(entry("llme_sigmoid_attention_finish")(ptr(partial), runs, ptr(gate), ld_gate, ptr(out), code(out.dtype), ld_out, T,
+                                                     heads, vdim, float(scale_out), stream()), "sigmoid_attention_finish")
+        return
     runs = max(1, min(64, (2 * compute_units()) // max(T, 1), (longest + 255) // 256))
     run_len = (longest + runs - 1) // runs
     run_len = (run_len + 31) // 32 * 32

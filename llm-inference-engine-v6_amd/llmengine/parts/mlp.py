@@ -60,13 +60,9 @@ class GatedMLP(FeedForward):
             ops.gemv_norm(x, weight, eps, self.w_gate_up, act, gated=True)
         else:
             act = step.buffer("mlp.act", (T, FF), x.dtype)
-            if self.activation == "silu":
-                ops.gemm_gated(x, self.w_gate_up, act, self.group,
-                               lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype), choices=step.choices)
-            else:
-                gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
-                ops.gemm(x, self.w_gate_up, gu, choices=step.choices)
-                ops.gated_activation(gu, act, self.group, self.activation)
+            ops.gemm_gated(x, self.w_gate_up, act, self.group,
+                           lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype), choices=step.choices,
+                           activation=self.activation)
         ops.gemm(act, self.w_down, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
 
 

@@ -54,11 +54,12 @@ class SigmoidAttention(ProjectedMixer):
         return []
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(kind="full", paged={"k": (self.kv_heads, PAGE, self.dim), "v": (self.kv_heads, PAGE, self.vdim)})
+        return CacheSpec(kind="full", paged={"k": (self.kv_heads, PAGE, self.dim), "v": (self.kv_heads, self.vdim, PAGE)})
 
     def load_core(self, get: Getter, placement: Placement) -> None:
         f32 = torch.float32
         self.talk = placement.place(get("talk"), f32)
+        self.talk_t = self.talk.t().contiguous()        # [from, to], as the matrix-core kernel reads it
         self.bias = placement.place(get("pb"), f32)
         if self.rot_dims:
             # frequencies in 64-bit, stored in 32-bit; the angle is the kernel's 32-bit product with the position
@@ -75,7 +76,7 @@ class SigmoidAttention(ProjectedMixer):
         q = step.buffer("sigmoid_attention.q", (T, n * dim), step.act_dtype)
         ops.rotate_write(p[:, :n_qkv], self.inv_freq, step, table, q, k_cache, v_cache, n, g, dim, vdim)
         ops.sigmoid_attention(q, k_cache, v_cache, self.talk, self.bias, p[:, n_qkv:n_qkv + n], step, table, o,
-                              n, g, dim, vdim, self.scale, scale)
+                              n, g, dim, vdim, self.scale, scale, mix_t=self.talk_t)
 
 
 register_part("mixer", "sigmoid_attention", SigmoidAttention)

@@ -192,6 +192,47 @@ def test_far_keys_and_page_borders_show_in_the_logits(tmp_path):
         assert _worst(got, {"r": ref}) < F32_TOL, sizes
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(8, 2, 64, 48), (16, 16, 32, 128), (4, 1, 128, 16)])
+def test_the_matrix_core_attention_agrees_with_the_plain_kernel(tmp_path, heads, kv_heads, dim, vdim):
+    """bfloat16 prompts take the matrix-core kernel of the attention without softmax, single tokens the plain one: the same
+    positions through both agree far below bfloat16's own rounding (they read the same rounded q, k and v and compute in
+    32-bit), and both are the plain model's within that rounding. Requests of 100, 16 and 37 rows in one step, portions
+    that start in the middle of a page, keys cut into several runs."""
+    cfg = rm.config([rm.parallel(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, rot_dims=32, scale=0.4, right_scale=0.0,
+                                 ff=None)], streams=None, width=64)
+    weights = _sharp_attention(cfg, rm.make_weights(cfg, 22, torch.bfloat16), far_scale=3.0)
+    engine, _ = _engine(tmp_path, cfg, 22, "bf16", weights=weights)
+    V = cfg["vocab"]
+    requests = {"a": _tokens(700, V, 1), "b": _tokens(16, V, 2), "c": _tokens(37, V, 3)}
+    ref = _reference(cfg, {k: v.float() for k, v in weights.items()}, requests)
+    from llmengine import StepEntry
+    cache = engine.new_cache(60, 16, 3)
+    for rid in requests:
+        cache.admit(rid)
+    fast = {}
+    rows = engine.step(cache, [StepEntry(rid, ids[:len(ids) // 2 + 3], list(range(len(ids) // 2 + 3)))
+                               for rid, ids in requests.items()]).cpu().numpy()
+    r = 0
+    for rid, ids in requests.items():
+        n = len(ids) // 2 + 3
+        fast[rid] = {p: rows[r + p].copy() for p in range(n)}
+        r += n
+    rows = engine.step(cache, [StepEntry(rid, ids[len(ids) // 2 + 3:], list(range(len(ids) - len(ids) // 2 - 3)))
+                               for rid, ids in requests.items() if len(ids) - len(ids) // 2 - 3 > 0]).cpu().numpy()
+    r = 0
+    for rid, ids in requests.items():
+        n0 = len(ids) // 2 + 3
+        for p in range(n0, len(ids)):
+            fast[rid][p] = rows[r].copy()
+            r += 1
+    for rid in requests:
+        cache.release(rid)
+    slow = replay.run_trace(engine, cache, replay.portions(requests, sizes=(7, 5, 15, 2, 11)))      # never 16 rows: the plain kernel
+    assert _covered(fast, requests) and _covered(slow, requests)
+    assert _worst(fast, {rid: np.stack([slow[rid][p] for p in range(len(ids))]) for rid, ids in requests.items()}) < 3e-3
+    assert _mean(fast, ref) < BF16_MEAN and _worst(fast, ref) < BF16_WORST
+
+
 def test_long_decoding_keeps_the_states(tmp_path):
     """300 tokens one by one after a short prompt (recorded decode steps replayed): the recurrent states and the
     convolutions' tails are carried in 32-bit without drift."""
