@@ -219,6 +219,14 @@ __global__ __launch_bounds__(256) void rglru_chunk_scan_kernel(const float* __re
     }
 }
 
+// dst [T, n] (contiguous) = src [T, n] with leading dimension ld: a few columns of a wide buffer made a matrix of their own.
+template <typename TO>
+__global__ __launch_bounds__(256) void copy_cols_kernel(const float* __restrict__ src, int ld, TO* __restrict__ dst, int n, size_t total) {
+    const size_t e = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= total) return;
+    dst[e] = from_float<TO>(src[(e / n) * ld + e % n]);
+}
+
 // ---------------------------------------------------------------------------------
 // x <- x / sqrt(sum(x^2) + eps) * scale over every head of `dim` entries, in place; heads [0, n_a) scale by
 // scale_a, heads [n_a, n_a + n_b) by scale_b (queries and keys lie side by side). One wavefront per (row, head).
@@ -238,6 +246,7 @@ __global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, 
 
 // beta[t, h] = sigmoid(b[t, h]);
 // per channel: decay[t, h, d] = exp(-exp(A_log[h]) softplus(sum_r a2[h dim + d, r] a1[t, r] + dt_bias[h dim + d]))
+//              (a2 null: a_in holds the sums already, [T, heads dim])
 // per head:    decay[t, h]    = exp(-exp(A_log[h]) softplus(a[t, h] + dt_bias[h]))
 template <typename TW>
 __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restrict__ b_in, int ld_b, const float* __restrict__ a_in,
@@ -252,7 +261,7 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
     if (e >= n_dec) return;
     const int h = per_channel ? e / dim : e;
     float z;
-    if (per_channel) {
+    if (per_channel && a2 != nullptr) {
         z = 0.f;
         const float* lo = a_in + static_cast<size_t>(t) * ld_a;
         const TW* row = a2 + static_cast<size_t>(e) * rank;
@@ -264,73 +273,138 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
     decay[static_cast<size_t>(t) * n_dec + e] = expf(-expf(A_log[h]) * softplusf_(z));
 }
 
-// The delta rule. State M [dim, vdim] per request and head (32-bit, in the request's slot). Per token:
+// The delta rule. State M per request and head (32-bit, in the request's slot), kept as [vdim][dim]: a column's key
+// channels lie together. Per token:
 //   M <- g * M (g per key channel or one per head);  w = beta (v - M^T k);  M <- M + k w^T;  o = M^T q.
-// The columns of M do not depend on each other: four lanes share a column (lane l holds the key channels
-// l, l + 4, ...), a workgroup of 256 threads owns 64 columns of one head of one request and walks the
-// request's rows in order. R = channels per lane.
+// The columns of M do not depend on each other: eight lanes share a column (lane l holds the R key channels l R ..
+// l R + R - 1), a workgroup of 256 threads owns 32 columns of one head of one request and walks the request's rows in
+// order. The rows' k, q, decay, v and beta come through LDS in blocks of eight rows, the next block asked for from
+// memory while the current one is worked through, so that a step waits for LDS only.
+constexpr int kDeltaCols = 32, kDeltaRows = 8, kDeltaFetch = 28;
+
+// The sum over each group of eight neighbouring lanes, in every lane of the group, by data-parallel-primitive moves
+// inside the vector unit (a shuffle through LDS would put three trips to LDS into every step of the recurrence):
+// neighbours in a quad, the quad's other pair, then the mirror image in the half row of 8.
+__device__ __forceinline__ float sum_of_8_lanes(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));     // quad_perm [1, 0, 3, 2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));     // quad_perm [2, 3, 0, 1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));    // row_half_mirror
+    return v;
+}
+
 template <int R, bool PER_CHANNEL>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int ld, int q_col, int k_col, int v_col,
                                                          const float* __restrict__ beta, const float* __restrict__ decay,
                                                          float* __restrict__ state, const int* __restrict__ q_start,
                                                          const int* __restrict__ slots, float* __restrict__ o, int heads,
                                                          int kv_heads, int dim, int vdim) {
-    const int s = blockIdx.z, h = blockIdx.y;
-    const int col = blockIdx.x * 64 + threadIdx.x / 4;
-    const int l = threadIdx.x % 4;
+    constexpr int DP = 8 * R;                               // a row's k (q, decay) padded with zeros to this many
+    constexpr int NV = PER_CHANNEL ? 3 : 2;
+    constexpr int W = NV * DP + kDeltaCols + 4;             // floats of a row in LDS: k, q, (decay,) v, beta, the head's decay
+    constexpr int BLOCK = kDeltaRows * W;
+    constexpr int NF = (BLOCK + 255) / 256;
+    static_assert(NF <= kDeltaFetch, "a block of rows is more than the threads fetch");
+    __shared__ float lds[2 * BLOCK];
+    const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kDeltaCols;
+    const int tid = threadIdx.x;
+    const int cl = tid / 8, l = tid % 8;
+    const int col = col0 + cl;
     const bool live = col < vdim;
     const int kvh = h / (heads / kv_heads);
     const int first = q_start[s], last = q_start[s + 1];
-    float* M = state + (static_cast<size_t>(slots[s]) * heads + h) * dim * vdim;
+    float* M = state + ((static_cast<size_t>(slots[s]) * heads + h) * vdim + (live ? col : 0)) * dim;
     float m[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int d = l + 4 * i;
-        m[i] = (live && d < dim) ? M[static_cast<size_t>(d) * vdim + col] : 0.f;
+        const int d = l * R + i;
+        m[i] = (live && d < dim) ? M[d] : 0.f;
     }
     const int n_dec = PER_CHANNEL ? heads * dim : heads;
-    for (int t = first; t < last; ++t) {
-        const float* row = qkv + static_cast<size_t>(t) * ld;
-        const float* kp = row + k_col + kvh * dim;
-        const float* qp = row + q_col + kvh * dim;
-        const float* gp = decay + static_cast<size_t>(t) * n_dec + (PER_CHANNEL ? h * dim : h);
-        const float bt = beta[static_cast<size_t>(t) * heads + h];
-        const float vv = live ? row[v_col + h * vdim + col] : 0.f;
-        float kk[R], qq[R];
-        const float g_head = PER_CHANNEL ? 1.f : gp[0];
-        float dot = 0.f;
+    float pre[NF];
+    auto fetch = [&](int t0) {
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int d = l + 4 * i;
-            const bool in = d < dim;
-            kk[i] = in ? kp[d] : 0.f;
-            qq[i] = in ? qp[d] : 0.f;
-            const float g = PER_CHANNEL ? (in ? gp[d] : 0.f) : g_head;
-            m[i] *= g;
-            dot += m[i] * kk[i];
+        for (int i = 0; i < NF; ++i) {
+            const int e = tid + 256 * i;
+            float val = 0.f;
+            if (e < BLOCK) {
+                const int tt = e / W, x = e % W, t = t0 + tt;
+                if (t < last) {
+                    const float* row = qkv + static_cast<size_t>(t) * ld;
+                    if (x < DP) {
+                        if (x < dim) val = row[k_col + kvh * dim + x];
+                    } else if (x < 2 * DP) {
+                        if (x - DP < dim) val = row[q_col + kvh * dim + x - DP];
+                    } else if (PER_CHANNEL && x < 3 * DP) {
+                        if (x - 2 * DP < dim) val = decay[static_cast<size_t>(t) * n_dec + h * dim + x - 2 * DP];
+                    } else {
+                        const int y = x - NV * DP;
+                        if (y < kDeltaCols) val = col0 + y < vdim ? row[v_col + h * vdim + col0 + y] : 0.f;
+                        else if (y == kDeltaCols) val = beta[static_cast<size_t>(t) * heads + h];
+                        else if (y == kDeltaCols + 1) val = PER_CHANNEL ? 1.f : decay[static_cast<size_t>(t) * heads + h];
+                    }
+                }
+            }
+            pre[i] = val;
         }
-        dot += __shfl_xor(dot, 1, kWave);
-        dot += __shfl_xor(dot, 2, kWave);
-        const float w = bt * (vv - dot);
-        float read = 0.f;
+    };
+    auto put = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            m[i] += kk[i] * w;
-            read += m[i] * qq[i];
+        for (int i = 0; i < NF; ++i) {
+            const int e = tid + 256 * i;
+            if (e < BLOCK) lds[buf * BLOCK + e] = pre[i];
         }
-        read += __shfl_xor(read, 1, kWave);
-        read += __shfl_xor(read, 2, kWave);
-        if (live && l == 0) o[static_cast<size_t>(t) * heads * vdim + h * vdim + col] = read;
+    };
+    fetch(first);
+    put(0);
+    __syncthreads();
+    int cur = 0;
+    for (int t0 = first; t0 < last; t0 += kDeltaRows) {
+        const bool more = t0 + kDeltaRows < last;
+        if (more) fetch(t0 + kDeltaRows);
+        const int nt = min(kDeltaRows, last - t0);
+        for (int tt = 0; tt < nt; ++tt) {
+            const float* row = lds + cur * BLOCK + tt * W;
+            const float* kp = row + l * R;
+            const float* qp = row + DP + l * R;
+            const float* gp = row + 2 * DP + l * R;
+            const float vv = row[NV * DP + cl];
+            const float bt = row[NV * DP + kDeltaCols];
+            const float g_head = row[NV * DP + kDeltaCols + 1];
+            float kk[R], qq[R];
+            float dots[2] = {0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                kk[i] = kp[i];
+                qq[i] = qp[i];
+                m[i] *= PER_CHANNEL ? gp[i] : g_head;
+                dots[i % 2] += m[i] * kk[i];
+            }
+            const float dot = sum_of_8_lanes(dots[0] + dots[1]);
+            const float w = bt * (vv - dot);
+            float reads[2] = {0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                m[i] += kk[i] * w;
+                reads[i % 2] += m[i] * qq[i];
+            }
+            const float read = sum_of_8_lanes(reads[0] + reads[1]);
+            if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read;
+        }
+        if (more) {
+            put(cur ^ 1);
+            __syncthreads();
+            cur ^= 1;
+        }
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int d = l + 4 * i;
-        if (live && d < dim) M[static_cast<size_t>(d) * vdim + col] = m[i];
+        const int d = l * R + i;
+        if (live && d < dim) M[d] = m[i];
     }
 }
 
 // out[t, h, j] = scale * o[t, h, j] / sqrt(mean_j o^2 + eps) * w[j] * gate, in the activation type.
-//   gate 0: sigmoid(sum_r g2[h vdim + j, r] g1[t, r]);  gate 1: silu(g[t, h vdim + j])
+//   gate 0: sigmoid(sum_r g2[h vdim + j, r] g1[t, r]);  gate 1: silu(g[t, h vdim + j]);  gate 2: sigmoid(g[t, h vdim + j])
 // One wavefront per (row, head).
 template <typename TW, typename TO>
 __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
@@ -349,7 +423,9 @@ __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __res
     const float* gi = g_in + static_cast<size_t>(t) * ld_g;
     for (int j = lane; j < vdim; j += kWave) {
         float z;
-        if (gate == 0) {
+        if (gate == 2) {
+            z = sigmoidf_(gi[h * vdim + j]);
+        } else if (gate == 0) {
             z = 0.f;
             const TW* row = g2 + static_cast<size_t>(h * vdim + j) * rank;
             for (int r = 0; r < rank; ++r) z += to_float(row[r]) * gi[r];
@@ -452,6 +528,19 @@ extern "C" int llme_rglru_scan_chunked(const void* decay, const void* drive, con
     return launch_status();
 }
 
+extern "C" int llme_copy_cols(const void* src, int ld, void* dst, int dst_dtype, int T, int n, hipStream_t stream) {
+    const size_t total = static_cast<size_t>(T) * n;
+    if (total == 0) return 0;
+    const int grid = static_cast<int>((total + 255) / 256);
+    if (dst_dtype == kF32)
+        copy_cols_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(src), ld, static_cast<float*>(dst), n, total);
+    else if (dst_dtype == kBF16)
+        copy_cols_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const float*>(src), ld, static_cast<bf16*>(dst), n, total);
+    else
+        return kErrBadArgument;
+    return launch_status();
+}
+
 extern "C" int llme_unit_heads(void* x, int ld, int T, int n_a, int n_b, int dim, float scale_a, float scale_b, float eps,
                                hipStream_t stream) {
     const long items = static_cast<long>(T) * (n_a + n_b);
@@ -487,23 +576,24 @@ static void launch_delta_rule(bool per_channel, dim3 grid, hipStream_t stream, c
 }
 
 // qkv [T, ld] 32-bit with unit q at q_col, unit k at k_col (kv_heads x dim each) and v at v_col (heads x vdim);
-// beta [T, heads]; decay [T, heads, dim] or [T, heads]; state [slots, heads, dim, vdim]; o [T, heads, vdim] 32-bit.
+// beta [T, heads]; decay [T, heads, dim] or [T, heads]; state [slots, heads, vdim, dim]; o [T, heads, vdim] 32-bit.
 extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, int v_col, const void* beta, const void* decay,
                                int per_channel, void* state, const void* q_start, const void* slots, void* o, int n_seq,
                                int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
     if (n_seq <= 0 || heads <= 0) return 0;
     if (kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return kErrBadArgument;
     if (dim > 256) return kErrUnsupported;
-    const dim3 grid((vdim + 63) / 64, heads, n_seq);
+    const dim3 grid((vdim + kDeltaCols - 1) / kDeltaCols, heads, n_seq);
 #define LLME_DELTA(R_)                                                                                                   \
     launch_delta_rule<R_>(per_channel != 0, grid, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col,      \
                           static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state), \
                           static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(o), heads, \
                           kv_heads, dim, vdim)
-    if (dim <= 32) LLME_DELTA(8);
-    else if (dim <= 64) LLME_DELTA(16);
-    else if (dim <= 128) LLME_DELTA(32);
-    else LLME_DELTA(64);
+    if (dim <= 16) LLME_DELTA(2);
+    else if (dim <= 32) LLME_DELTA(4);
+    else if (dim <= 64) LLME_DELTA(8);
+    else if (dim <= 128) LLME_DELTA(16);
+    else LLME_DELTA(32);
 #undef LLME_DELTA
     return launch_status();
 }

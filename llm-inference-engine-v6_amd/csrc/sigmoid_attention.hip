@@ -164,7 +164,7 @@ __global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r16 = lane % 16, q4 = lane / 16;
     // which request and which 16 of its rows
-    int item = blockIdx.x, s = 0, row0 = 0, nrows = 0;
+    int item = gridDim.x - 1 - blockIdx.x, s = 0, row0 = 0, nrows = 0;       // (later rows have more keys: they start first)
     for (; s < n_seq; ++s) {
         const int n = q_start[s + 1] - q_start[s];
         const int tiles = (n + 15) / 16;

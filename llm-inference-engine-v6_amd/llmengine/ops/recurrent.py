@@ -30,6 +30,7 @@ declare("llme_short_conv", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i,
 declare("llme_rglru_gates", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp])
 declare("llme_rglru_scan", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
 declare("llme_rglru_scan_chunked", [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp])
+declare("llme_copy_cols", [_vp, _i, _vp, _i, _i, _i, _vp])
 declare("llme_unit_heads", [_vp, _i, _i, _i, _i, _i, _f, _f, _f, _vp])
 declare("llme_delta_gates", [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp])
 declare("llme_delta_rule", [_vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
@@ -191,6 +192,14 @@ def rglru_scan(decay: torch.Tensor, drive: torch.Tensor, y: torch.Tensor, y_bias
 
 
 # --- gated delta rule ----------------------------------------------------------------------
+def copy_cols(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst [T, n] (contiguous, 32-bit or bfloat16) = src [T, n], a column range of a wider 32-bit buffer."""
+    T, n = src.shape
+    ld = _cols(src, "src", torch.float32)
+    require(dst, "dst", _FLOATS, (T, n))
+    check(entry("llme_copy_cols")(ptr(src), ld, ptr(dst), code(dst.dtype), T, n, stream()), "copy_cols")
+
+
 def unit_heads(x: torch.Tensor, n_a: int, n_b: int, dim: int, scale_a: float, scale_b: float, eps: float) -> None:
     """In place: every head of `dim` entries of x [T, (n_a + n_b) dim] becomes x / sqrt(sum(x^2) + eps), times
     scale_a for the first n_a heads and scale_b for the rest."""
@@ -202,31 +211,33 @@ def unit_heads(x: torch.Tensor, n_a: int, n_b: int, dim: int, scale_a: float, sc
 
 def delta_gates(b_in: torch.Tensor, a_in: torch.Tensor, a2: torch.Tensor | None, A_log: torch.Tensor, dt_bias: torch.Tensor,
                 beta: torch.Tensor, decay: torch.Tensor, heads: int, dim: int) -> None:
-    """beta = sigmoid(b_in) [T, heads]; decay = exp(-exp(A_log[head]) * softplus(z + dt_bias)) with, per key channel
-    (a2 [heads * dim, rank] given), z = a_in a2^T and decay [T, heads * dim], or per head, z = a_in and decay [T, heads]."""
+    """beta = sigmoid(b_in) [T, heads]; decay = exp(-exp(A_log[head]) * softplus(z + dt_bias)) with, per key channel,
+    z = a_in a2^T (a2 [heads * dim, rank] given) or z = a_in [T, heads * dim] (a2 None) and decay [T, heads * dim], or per
+    head, z = a_in [T, heads] and decay [T, heads]; which of the last two, the shape of `decay` says."""
     T = b_in.shape[0]
     ld_b = _cols(b_in, "b_in", torch.float32, T, heads)
-    per_channel = a2 is not None
+    per_channel = a2 is not None or decay.shape[1] == heads * dim and a_in.shape[1] == heads * dim and dim > 1
     n = heads * dim if per_channel else heads
     rank = 0
-    if per_channel:
+    if a2 is not None:
         require(a2, "a2", _FLOATS, (n, None))
         rank = a2.shape[1]
         ld_a = _cols(a_in, "a_in", torch.float32, T, rank)
     else:
-        ld_a = _cols(a_in, "a_in", torch.float32, T, heads)
+        ld_a = _cols(a_in, "a_in", torch.float32, T, n)
     require(A_log, "A_log", torch.float32, (heads,))
     require(dt_bias, "dt_bias", torch.float32, (n,))
     require(beta, "beta", torch.float32, (T, heads))
     require(decay, "decay", torch.float32, (T, n))
     check(entry("llme_delta_gates")(ptr(b_in), ld_b, ptr(a_in), ld_a, ptr(a2), rank, ptr(A_log), ptr(dt_bias),
-                                    code(a2.dtype) if per_channel else 0, ptr(beta), ptr(decay), T, heads, dim,
+                                    code(a2.dtype) if a2 is not None else 0, ptr(beta), ptr(decay), T, heads, dim,
                                     1 if per_channel else 0, stream()), "delta_gates")
 
 
 def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, step, o: torch.Tensor,
                heads: int, kv_heads: int, dim: int, vdim: int, per_channel: bool) -> None:
-    """The delta rule over each request's rows, from and into its slot of state [slots, heads, dim, vdim]:
+    """The delta rule over each request's rows, from and into its slot of state [slots, heads, vdim, dim] (M transposed:
+    a column's key channels lie together):
     M <- decay * M; w = beta (v - M^T k); M <- M + k w^T; o = M^T q. qkv [T, (2 kv_heads dim + heads vdim)] holds
     unit q, unit k and v side by side; decay is [T, heads * dim] (per key channel) or [T, heads]."""
     T = qkv.shape[0]
@@ -239,7 +250,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
     require(decay, "decay", torch.float32, (T, None))
     if decay.shape[1] != (heads * dim if per_channel else heads):
         raise KernelError(f"delta_rule: decay has {decay.shape[1]} columns for {heads} heads of {dim}")
-    require(state, "state", torch.float32, (None, heads, dim, vdim))
+    require(state, "state", torch.float32, (None, heads, vdim, dim))
     require(o, "o", torch.float32, (T, heads * vdim))
     if T != step.num_tokens:
         raise KernelError("delta_rule: one row per token of the step")
@@ -249,9 +260,10 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
 
 
 def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate_in: torch.Tensor, g2: torch.Tensor | None, out: torch.Tensor,
-                    heads: int, vdim: int, eps: float, scale: float = 1.0) -> None:
+                    heads: int, vdim: int, eps: float, scale: float = 1.0, activation: str = "silu") -> None:
     """out = scale * o / sqrt(mean(o^2) + eps) * weight * gate over every head of o [T, heads * vdim];
-    gate = sigmoid(gate_in g2^T) where g2 [heads * vdim, rank] is given, else silu(gate_in)."""
+    gate = sigmoid(gate_in g2^T) where g2 [heads * vdim, rank] is given, else silu(gate_in) or (activation "sigmoid")
+    sigmoid(gate_in) with gate_in [T, heads * vdim]."""
     T = o.shape[0]
     require(o, "o", torch.float32, (T, heads * vdim))
     require(weight, "weight", torch.float32, (vdim,))
@@ -263,7 +275,8 @@ def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate_in: torch.Tensor
     else:
         ld_g = _cols(gate_in, "gate_in", torch.float32, T, heads * vdim)
     ld_out = _cols(out, "out", _FLOATS, T, heads * vdim)
-    check(entry("llme_gated_head_norm")(ptr(o), ptr(weight), ptr(gate_in), ld_g, ptr(g2), rank, 0 if g2 is not None else 1,
+    check(entry("llme_gated_head_norm")(ptr(o), ptr(weight), ptr(gate_in), ld_g, ptr(g2), rank,
+                                        0 if g2 is not None else (2 if activation == "sigmoid" else 1),
                                         code(g2.dtype) if g2 is not None else 0, ptr(out), code(out.dtype), ld_out, T, heads,
                                         vdim, float(eps), float(scale), stream()), "gated_head_norm")
 
@@ -305,9 +318,6 @@ def sigmoid_attention_mfma_fits(q: torch.Tensor, heads: int, dim: int, vdim: int
             and vdim % 16 == 0 and vdim <= 128 and page % 16 == 0)
 
 
-SIGMOID_ATTENTION_MFMA_ROWS = 16        # a request must bring this many rows for the step to take the matrix-core kernel
-
-
 def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, mix: torch.Tensor, bias: torch.Tensor,
                       gate: torch.Tensor, step, block_table: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                       dim: int, vdim: int, scale: float, scale_out: float = 1.0, mix_t: torch.Tensor | None = None) -> None:
@@ -333,12 +343,15 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         longest = max(c + n for c, n in zip(step.ctx_lens, step.new_lens))
     from .mfma import compute_units
     from .choices import choices_of
-    if (step.plan_len is None and mix_t is not None and choices_of(step).fast_attention
-            and max(step.new_lens) >= SIGMOID_ATTENTION_MFMA_ROWS and sigmoid_attention_mfma_fits(q, heads, dim, vdim, page)):
-        # prompts and their portions: 16 rows of a request to a workgroup, scores and the second product on the matrix cores
+    if (mix_t is not None and choices_of(step).fast_attention and sigmoid_attention_mfma_fits(q, heads, dim, vdim, page)):
+        # up to 16 rows of a request to a workgroup, scores and the second product on the matrix cores; single decoded
+        # tokens too (a tile of one row wastes matrix work, which is cheap; what counts there is that the keys are read
+        # in whole lines and cut into enough runs to fill the chip). The grid follows the step's shape only (a recorded
+        # step plans for the longest request its block tables hold).
         require(mix_t, "mix_t", torch.float32, (heads, heads))
         tiles = sum((n + 15) // 16 for n in step.new_lens)
-        runs = max(1, min(32, (2 * compute_units()) // tiles, (longest + 511) // 512))
+        shortest_run = 256 if tiles >= 32 else 64
+        runs = max(1, min(64, -(-4 * compute_units() // tiles), (longest + shortest_run - 1) // shortest_run))
         run_len = ((longest + runs - 1) // runs + 31) // 32 * 32
         runs = max(1, (longest + run_len - 1) // run_len)
         partial = step.buffer("sigmoid_attention.partial", (runs, T, heads * vdim), torch.float32)

@@ -89,7 +89,7 @@ class GatedDeltaRule(ProjectedMixer):
         return out
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(state={"memory": ((self.heads, self.dim, self.vdim), torch.float32),
+        return CacheSpec(state={"memory": ((self.heads, self.vdim, self.dim), torch.float32),
                                 "conv": ((max(self.taps - 1, 0), self.conv_channels), torch.float32)})
 
     def load_core(self, get: Getter, placement: Placement) -> None:
@@ -128,11 +128,23 @@ class GatedDeltaRule(ProjectedMixer):
         beta = step.buffer("delta.beta", (T, heads), torch.float32)
         n_dec = heads * dim if self.decay == "channel" else heads
         decay = step.buffer("delta.decay", (T, n_dec), torch.float32)
-        ops.delta_gates(b_in, a_in, self.a2, self.A_log, self.dt_bias, beta, decay, heads, dim)
+        if self.a2 is not None:
+            # the second stage of the two-stage map as a product of its own, its 32-bit input made contiguous first
+            low = step.buffer("delta.decay_low", (T, self.decay_rank), torch.float32)
+            ops.copy_cols(a_in, low)
+            a_in = step.buffer("delta.decay_in", (T, n_dec), torch.float32)
+            ops.gemm(low, self.a2, a_in, choices=step.choices)
+        ops.delta_gates(b_in, a_in, None, self.A_log, self.dt_bias, beta, decay, heads, dim)
         read = step.buffer("delta.read", (T, heads * vdim), torch.float32)
         ops.delta_rule(qkv, beta, decay, cache.state["memory"], step, read, heads, kvh, dim, vdim,
                        per_channel=self.decay == "channel")
-        ops.gated_head_norm(read, self.norm_w, g_in, self.g2, o, heads, vdim, self.eps, scale)
+        if self.g2 is not None:
+            low = step.buffer("delta.gate_low", (T, self.gate_rank), torch.float32)
+            ops.copy_cols(g_in, low)
+            g_in = step.buffer("delta.gate_in", (T, heads * vdim), torch.float32)
+            ops.gemm(low, self.g2, g_in, choices=step.choices)
+        ops.gated_head_norm(read, self.norm_w, g_in, None, o, heads, vdim, self.eps, scale,
+                            activation="sigmoid" if self.gate == "sigmoid_lowrank" else "silu")
 
 
 register_part("mixer", "gated_delta", GatedDeltaRule)

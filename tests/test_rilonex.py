@@ -77,7 +77,7 @@ def test_a_rank_left_to_the_checkpoint_fits_any_size():
 def test_the_cache_spec_of_every_mixer():
     specs = _model(rm.MIXED).cache_specs()
     assert set(specs[0].state) == {"s", "conv"} and specs[0].state["conv"][0] == (2, 48) and not specs[0].paged
-    assert specs[1].state["memory"][0] == (4, 24, 20) and specs[1].state["conv"][0] == (3, 2 * 48 + 80)
+    assert specs[1].state["memory"][0] == (4, 20, 24) and specs[1].state["conv"][0] == (3, 2 * 48 + 80)
     assert set(specs[2].paged) == {"left.k", "left.v"} and set(specs[2].state) == {"right.memory", "right.conv"}
     assert all(dtype == torch.float32 for spec in specs.values() for _, dtype in spec.state.values())
 

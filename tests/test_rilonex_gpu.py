@@ -194,7 +194,7 @@ def test_far_keys_and_page_borders_show_in_the_logits(tmp_path):
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(8, 2, 64, 48), (16, 16, 32, 128), (4, 1, 128, 16)])
 def test_the_matrix_core_attention_agrees_with_the_plain_kernel(tmp_path, heads, kv_heads, dim, vdim):
-    """bfloat16 prompts take the matrix-core kernel of the attention without softmax, single tokens the plain one: the same
+    """bfloat16 steps take the matrix-core kernel of the attention without softmax unless an engine is told not to: the same
     positions through both agree far below bfloat16's own rounding (they read the same rounded q, k and v and compute in
     32-bit), and both are the plain model's within that rounding. Requests of 100, 16 and 37 rows in one step, portions
     that start in the middle of a page, keys cut into several runs."""
@@ -227,7 +227,11 @@ def test_the_matrix_core_attention_agrees_with_the_plain_kernel(tmp_path, heads,
             r += 1
     for rid in requests:
         cache.release(rid)
-    slow = replay.run_trace(engine, cache, replay.portions(requests, sizes=(7, 5, 15, 2, 11)))      # never 16 rows: the plain kernel
+    from llmengine.ops import KernelChoices
+    plain_engine, _ = _engine(tmp_path / "plain", cfg, 22, "bf16", weights=weights, kernel_choices=KernelChoices(fast_attention=False))
+    slow = replay.run_trace(plain_engine, plain_engine.new_cache(60, 16, 3), replay.portions(requests, sizes=(7, 5, 15, 2, 11)))
+    small = replay.run_trace(engine, cache, replay.portions(requests, sizes=(1, 3, 16, 2, 40)))      # tiles of a few rows
+    assert _worst(small, {rid: np.stack([slow[rid][p] for p in range(len(ids))]) for rid, ids in requests.items()}) < 3e-3
     assert _covered(fast, requests) and _covered(slow, requests)
     assert _worst(fast, {rid: np.stack([slow[rid][p] for p in range(len(ids))]) for rid, ids in requests.items()}) < 3e-3
     assert _mean(fast, ref) < BF16_MEAN and _worst(fast, ref) < BF16_WORST
