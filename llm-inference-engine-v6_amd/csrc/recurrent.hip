@@ -362,21 +362,44 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         const bool more = t0 + kDeltaRows < last;
         if (more) fetch(t0 + kDeltaRows);
         const int nt = min(kDeltaRows, last - t0);
-        for (int tt = 0; tt < nt; ++tt) {
+#pragma unroll
+        for (int tt = 0; tt < kDeltaRows; ++tt) {
+            if (tt >= nt) break;
             const float* row = lds + cur * BLOCK + tt * W;
-            const float* kp = row + l * R;
-            const float* qp = row + DP + l * R;
-            const float* gp = row + 2 * DP + l * R;
             const float vv = row[NV * DP + cl];
             const float bt = row[NV * DP + kDeltaCols];
             const float g_head = row[NV * DP + kDeltaCols + 1];
-            float kk[R], qq[R];
+            float kk[R], qq[R], gg[R];
+            // a lane's R channels of k, q and the decay lie together and aligned: whole vectors from LDS
+            if constexpr (R % 4 == 0) {
+#pragma unroll
+                for (int i = 0; i < R; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(row + l * R + i);
+                    const float4 q4v = *reinterpret_cast<const float4*>(row + DP + l * R + i);
+                    kk[i] = k4.x; kk[i + 1] = k4.y; kk[i + 2] = k4.z; kk[i + 3] = k4.w;
+                    qq[i] = q4v.x; qq[i + 1] = q4v.y; qq[i + 2] = q4v.z; qq[i + 3] = q4v.w;
+                    if (PER_CHANNEL) {
+                        const float4 g4 = *reinterpret_cast<const float4*>(row + 2 * DP + l * R + i);
+                        gg[i] = g4.x; gg[i + 1] = g4.y; gg[i + 2] = g4.z; gg[i + 3] = g4.w;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; i += 2) {
+                    const float2 k2 = *reinterpret_cast<const float2*>(row + l * R + i);
+                    const float2 q2 = *reinterpret_cast<const float2*>(row + DP + l * R + i);
+                    kk[i] = k2.x; kk[i + 1] = k2.y;
+                    qq[i] = q2.x; qq[i + 1] = q2.y;
+                    if (PER_CHANNEL) {
+                        const float2 g2 = *reinterpret_cast<const float2*>(row + 2 * DP + l * R + i);
+                        gg[i] = g2.x; gg[i + 1] = g2.y;
+                    }
+                }
+            }
             float dots[2] = {0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                kk[i] = kp[i];
-                qq[i] = qp[i];
-                m[i] *= PER_CHANNEL ? gp[i] : g_head;
+                m[i] *= PER_CHANNEL ? gg[i] : g_head;
                 dots[i % 2] += m[i] * kk[i];
             }
             const float dot = sum_of_8_lanes(dots[0] + dots[1]);

@@ -197,22 +197,43 @@ __global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
 #pragma unroll
         for (int dt = 0; dt < VT; ++dt) o[hh][dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
+    // The wavefront's four heads read one key/value head where the query heads come four or more to one (ONE_KV): its
+    // keys for the next tile are then asked for as soon as this tile's scores are made, and its values ahead of the scores.
+    const bool one_kv = (h0 / per) == ((h0 + HPW - 1) / per);
+    sa_bf16x8 kf[2][DIM32], vf[VT];
+    auto load_k = [&](int j, int kv) {
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int key = min(j + rt * 16 + r16, kmax);
+            const bf16* kp = k_cache + ((static_cast<size_t>(table[key / page]) * G + kv) * page + key % page) * DIM;
+#pragma unroll
+            for (int c = 0; c < DIM32; ++c) kf[rt][c] = *reinterpret_cast<const sa_bf16x8*>(kp + c * 32 + q4 * 8);
+        }
+    };
+    auto load_v = [&](int j, int kv) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int key = min(j + half * 16 + 4 * q4, kmax & ~3);
+            const bf16* vp = v_cache + (static_cast<size_t>(table[key / page]) * G + kv) * VDIM * page + key % page;
+#pragma unroll
+            for (int dt = 0; dt < VT; ++dt) {
+                const sa_bf16x4 v4 = *reinterpret_cast<const sa_bf16x4*>(vp + static_cast<size_t>(dt * 16 + r16) * page);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vf[dt][half * 4 + e] = v4[e];
+            }
+        }
+    };
+    if (one_kv && key_lo < key_hi) load_k(key_lo, h0 / per);
     for (int j0 = key_lo; j0 < key_hi; j0 += 32) {
         // (1) transposed scores of this wavefront's heads
         {
-            int have = -1;
-            sa_bf16x8 kf[2][DIM32];
+            int have = one_kv ? h0 / per : -1;
+            if (one_kv) load_v(j0, h0 / per);
 #pragma unroll
             for (int hh = 0; hh < HPW; ++hh) {
                 const int g = h0 + hh, kv = g / per;
                 if (kv != have) {
-#pragma unroll
-                    for (int rt = 0; rt < 2; ++rt) {
-                        const int key = min(j0 + rt * 16 + r16, kmax);
-                        const bf16* kp = k_cache + ((static_cast<size_t>(table[key / page]) * G + kv) * page + key % page) * DIM;
-#pragma unroll
-                        for (int c = 0; c < DIM32; ++c) kf[rt][c] = *reinterpret_cast<const sa_bf16x8*>(kp + c * 32 + q4 * 8);
-                    }
+                    load_k(j0, kv);
                     have = kv;
                 }
                 sa_f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
@@ -225,6 +246,7 @@ __global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
                 *reinterpret_cast<float4*>(dst) = float4{a0[0] * scale, a0[1] * scale, a0[2] * scale, a0[3] * scale};
                 *reinterpret_cast<float4*>(dst + 4) = float4{a1[0] * scale, a1[1] * scale, a1[2] * scale, a1[3] * scale};
             }
+            if (one_kv && j0 + 32 < key_hi) load_k(j0 + 32, h0 / per);
         }
         __syncthreads();
         // (2) all heads' scores mixed into this wavefront's heads
@@ -245,8 +267,7 @@ __global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
                 for (int e = 0; e < 8; ++e) m[hh][e] += tv[hh] * sv[e];
         }
         {
-            int have = -1;
-            sa_bf16x8 vf[VT];
+            int have = one_kv ? h0 / per : -1;
 #pragma unroll
             for (int hh = 0; hh < HPW; ++hh) {
                 const int h = h0 + hh, kv = h / per;
@@ -260,17 +281,7 @@ __global__ __launch_bounds__(512) void sigmoid_attention_mfma_kernel(
                     lo[e] = static_cast<__bf16>(w - static_cast<float>(hi[e]));
                 }
                 if (kv != have) {
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        const int key = min(j0 + half * 16 + 4 * q4, kmax & ~3);
-                        const bf16* vp = v_cache + (static_cast<size_t>(table[key / page]) * G + kv) * VDIM * page + key % page;
-#pragma unroll
-                        for (int dt = 0; dt < VT; ++dt) {
-                            const sa_bf16x4 v4 = *reinterpret_cast<const sa_bf16x4*>(vp + static_cast<size_t>(dt * 16 + r16) * page);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) vf[dt][half * 4 + e] = v4[e];
-                        }
-                    }
+                    load_v(j0, kv);
                     have = kv;
                 }
 #pragma unroll
@@ -322,7 +333,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_finish_kernel(const flo
                                                                        float scale_out) {
     const int t = blockIdx.x;
     const size_t per_run = static_cast<size_t>(T) * H * vdim;
-    for (int e = threadIdx.x; e < H * vdim; e += 256) {
+    for (int e = blockIdx.y * 256 + threadIdx.x; e < H * vdim; e += gridDim.y * 256) {
         float a = 0.f;
         for (int r = 0; r < runs; ++r) a += partial[r * per_run + static_cast<size_t>(t) * H * vdim + e];
         const float g = 1.0f / (1.0f + expf(-gate[static_cast<size_t>(t) * ld_gate + e / vdim]));
@@ -437,11 +448,11 @@ extern "C" int llme_sigmoid_attention_finish(const void* partial, int runs, cons
                                              int ld_out, int T, int H, int vdim, float scale_out, hipStream_t stream) {
     if (T <= 0) return 0;
     if (out_dtype == kF32)
-        sigmoid_attention_finish_kernel<float><<<T, 256, 0, stream>>>(static_cast<const float*>(partial), runs,
+        sigmoid_attention_finish_kernel<float><<<dim3(T, (H * vdim + 255) / 256), 256, 0, stream>>>(static_cast<const float*>(partial), runs,
                                                                       static_cast<const float*>(gate), ld_gate,
                                                                       static_cast<float*>(out), ld_out, T, H, vdim, scale_out);
     else if (out_dtype == kBF16)
-        sigmoid_attention_finish_kernel<bf16><<<T, 256, 0, stream>>>(static_cast<const float*>(partial), runs,
+        sigmoid_attention_finish_kernel<bf16><<<dim3(T, (H * vdim + 255) / 256), 256, 0, stream>>>(static_cast<const float*>(partial), runs,
                                                                      static_cast<const float*>(gate), ld_gate,
                                                                      static_cast<bf16*>(out), ld_out, T, H, vdim, scale_out);
     else

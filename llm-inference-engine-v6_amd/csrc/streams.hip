@@ -19,12 +19,6 @@ __global__ __launch_bounds__(256) void streams_spread_kernel(float4* __restrict_
     }
 }
 
-struct StreamWeights {
-    float in[kMaxStreams];
-    float out[kMaxStreams];
-    float mix[kMaxStreams * kMaxStreams];
-};
-
 // One workgroup per output row. The row's mixed value is kept in registers between the two passes
 // (up to NV values per thread), or recomputed when the row is wider than that.
 template <typename TW, typename TO, int NV>
@@ -83,6 +77,60 @@ __global__ __launch_bounds__(256) void streams_read_norm_kernel(const float* __r
     }
 }
 
+// The same with a row's values four at a time (H a multiple of 4, at most 1024 NV4): every load of a thread is asked
+// for before the first is used, so that a step of a few rows (decoding) does not wait for them one after the other.
+constexpr int kVecStreams = 4;     // streams the vector form holds in registers
+template <typename TW, typename TO, int NV4>
+__global__ __launch_bounds__(256) void streams_read_norm_vec_kernel(const float* __restrict__ x, int S, size_t stream_stride,
+                                                                     const float* __restrict__ a, const TW* __restrict__ w,
+                                                                     TO* __restrict__ out, const int* __restrict__ rows,
+                                                                     int H, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    const float* xr = x + static_cast<size_t>(src) * H;
+    float coef[kVecStreams];
+#pragma unroll
+    for (int s = 0; s < kVecStreams; ++s) coef[s] = s < S ? (a ? a[s] : 1.0f) : 0.f;
+    float4 v[NV4][kVecStreams];
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        const int i = (threadIdx.x + j * 256) * 4;
+#pragma unroll
+        for (int s = 0; s < kVecStreams; ++s)
+            v[j][s] = (i < H && s < S) ? *reinterpret_cast<const float4*>(xr + static_cast<size_t>(s) * stream_stride + i)
+                                       : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float u[NV4][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        u[j][0] = u[j][1] = u[j][2] = u[j][3] = 0.f;
+#pragma unroll
+        for (int s = 0; s < kVecStreams; ++s) {
+            u[j][0] += coef[s] * v[j][s].x;
+            u[j][1] += coef[s] * v[j][s].y;
+            u[j][2] += coef[s] * v[j][s].z;
+            u[j][3] += coef[s] * v[j][s].w;
+        }
+        ss += u[j][0] * u[j][0] + u[j][1] * u[j][1] + u[j][2] * u[j][2] + u[j][3] * u[j][3];
+    }
+    TO* o = out + static_cast<size_t>(r) * H;
+    float inv = 1.f;
+    if (w != nullptr) {
+        ss = block_sum(ss, scratch, 4);
+        inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+    }
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        const int i = (threadIdx.x + j * 256) * 4;
+        if (i >= H) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            o[i + e] = from_float<TO>(w != nullptr ? (to_float(w[i + e]) * u[j][e]) * inv : u[j][e]);
+    }
+}
+
 __global__ __launch_bounds__(256) void streams_write_kernel(float* __restrict__ x, int S, size_t n, const float* __restrict__ mix,
                                                             const float* __restrict__ b, const float* __restrict__ y) {
     __shared__ float m[kMaxStreams * kMaxStreams];
@@ -112,6 +160,12 @@ static int launch_read_norm(const float* x, int S, size_t stride, const float* a
                             int R, int H, float eps, hipStream_t stream) {
     const TW* wp = static_cast<const TW*>(w);
     TO* op = static_cast<TO*>(out);
+    if (H % 4 == 0 && H <= 4096 && S <= kVecStreams && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        if (H <= 1024) streams_read_norm_vec_kernel<TW, TO, 1><<<R, 256, 0, stream>>>(x, S, stride, a, wp, op, rows, H, eps);
+        else if (H <= 2048) streams_read_norm_vec_kernel<TW, TO, 2><<<R, 256, 0, stream>>>(x, S, stride, a, wp, op, rows, H, eps);
+        else streams_read_norm_vec_kernel<TW, TO, 4><<<R, 256, 0, stream>>>(x, S, stride, a, wp, op, rows, H, eps);
+        return launch_status();
+    }
     if (H <= 1024)
         streams_read_norm_kernel<TW, TO, 4><<<R, 256, 0, stream>>>(x, S, stride, a, wp, op, rows, H, eps);
     else
