@@ -320,31 +320,46 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         m[i] = (live && d < dim) ? M[d] : 0.f;
     }
     const int n_dec = PER_CHANNEL ? heads * dim : heads;
+    // Where each of a thread's NF values of a block of rows comes from is the same for every block: the address for the
+    // first block and the distance to the next block's are worked out once (src null: padding, always zero).
     float pre[NF];
+    const float* src[NF];
+    int advance[NF], row_of[NF];
+#pragma unroll
+    for (int i = 0; i < NF; ++i) {
+        const int e = tid + 256 * i;
+        src[i] = nullptr;
+        advance[i] = 0;
+        row_of[i] = 0;
+        if (e < BLOCK) {
+            const int tt = e / W, x = e % W;
+            const size_t t = static_cast<size_t>(first + tt);
+            row_of[i] = tt;
+            if (x < DP) {
+                if (x < dim) { src[i] = qkv + t * ld + k_col + kvh * dim + x; advance[i] = kDeltaRows * ld; }
+            } else if (x < 2 * DP) {
+                if (x - DP < dim) { src[i] = qkv + t * ld + q_col + kvh * dim + x - DP; advance[i] = kDeltaRows * ld; }
+            } else if (PER_CHANNEL && x < 3 * DP) {
+                if (x - 2 * DP < dim) { src[i] = decay + t * n_dec + h * dim + x - 2 * DP; advance[i] = kDeltaRows * n_dec; }
+            } else {
+                const int y = x - NV * DP;
+                if (y < kDeltaCols) {
+                    if (col0 + y < vdim) { src[i] = qkv + t * ld + v_col + h * vdim + col0 + y; advance[i] = kDeltaRows * ld; }
+                } else if (y == kDeltaCols) {
+                    src[i] = beta + t * heads + h;
+                    advance[i] = kDeltaRows * heads;
+                } else if (y == kDeltaCols + 1 && !PER_CHANNEL) {
+                    src[i] = decay + t * heads + h;
+                    advance[i] = kDeltaRows * heads;
+                }
+            }
+        }
+    }
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < NF; ++i) {
-            const int e = tid + 256 * i;
-            float val = 0.f;
-            if (e < BLOCK) {
-                const int tt = e / W, x = e % W, t = t0 + tt;
-                if (t < last) {
-                    const float* row = qkv + static_cast<size_t>(t) * ld;
-                    if (x < DP) {
-                        if (x < dim) val = row[k_col + kvh * dim + x];
-                    } else if (x < 2 * DP) {
-                        if (x - DP < dim) val = row[q_col + kvh * dim + x - DP];
-                    } else if (PER_CHANNEL && x < 3 * DP) {
-                        if (x - 2 * DP < dim) val = decay[static_cast<size_t>(t) * n_dec + h * dim + x - 2 * DP];
-                    } else {
-                        const int y = x - NV * DP;
-                        if (y < kDeltaCols) val = col0 + y < vdim ? row[v_col + h * vdim + col0 + y] : 0.f;
-                        else if (y == kDeltaCols) val = beta[static_cast<size_t>(t) * heads + h];
-                        else if (y == kDeltaCols + 1) val = PER_CHANNEL ? 1.f : decay[static_cast<size_t>(t) * heads + h];
-                    }
-                }
-            }
-            pre[i] = val;
+            pre[i] = (src[i] != nullptr && t0 + row_of[i] < last) ? *src[i] : 0.f;
+            if (src[i] != nullptr) src[i] += advance[i];
         }
     };
     auto put = [&](int buf) {
