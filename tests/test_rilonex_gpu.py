@@ -67,6 +67,8 @@ ONE_LAYER = {
     "parallel_right_only": rm.config([rm.parallel(left_scale=0.0, ff=None)], streams=None),
     "feed_forward_and_streams": rm.config([rm.rglru(width=16, blocks=2, ff=56)], streams=4),
     "one_stream": rm.config([rm.channel_delta(ff=32)], streams=1),
+    "one_tap_and_wide_keys": rm.config([rm.channel_delta(heads=2, kv_heads=1, dim=136, vdim=8, conv=1, ff=None),
+                                        rm.rglru(width=24, blocks=2, conv=1, ff=None)], streams=None),
 }
 
 
