@@ -276,29 +276,34 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
 // The delta rule. State M per request and head (32-bit, in the request's slot), kept as [vdim][dim]: a column's key
 // channels lie together. Per token:
 //   M <- g * M (g per key channel or one per head);  w = beta (v - M^T k);  M <- M + k w^T;  o = M^T q.
-// The columns of M do not depend on each other: eight lanes share a column (lane l holds the R key channels l R ..
-// l R + R - 1), a workgroup of 256 threads owns 32 columns of one head of one request and walks the request's rows in
-// order. The rows' k, q, decay, v and beta come through LDS in blocks of eight rows, the next block asked for from
+// The columns of M do not depend on each other: LPC lanes (8, or 16 for keys of 64 and more) share a column (lane l holds
+// the R key channels l R .. l R + R - 1), a workgroup of 256 threads owns 256 / LPC columns of one head of one request and
+// walks the request's rows in order: the fewer channels a lane holds, the shorter a step, and a prompt's time is its steps'. The rows' k, q, decay, v and beta come through LDS in blocks of eight rows, the next block asked for from
 // memory while the current one is worked through, so that a step waits for LDS only.
-constexpr int kDeltaCols = 32, kDeltaRows = 8, kDeltaFetch = 28;
+constexpr int kDeltaRows = 8, kDeltaFetch = 28;
 
-// The sum over each group of eight neighbouring lanes, in every lane of the group, by data-parallel-primitive moves
+// The sum over each group of 8 or 16 neighbouring lanes, in every lane of the group, by data-parallel-primitive moves
 // inside the vector unit (a shuffle through LDS would put three trips to LDS into every step of the recurrence):
 // neighbours in a quad, the quad's other pair, then the mirror image in the half row of 8.
-__device__ __forceinline__ float sum_of_8_lanes(float v) {
+template <int LANES>
+__device__ __forceinline__ float sum_of_lanes(float v) {
+    static_assert(LANES == 8 || LANES == 16, "groups of 8 or 16 lanes");
     v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));     // quad_perm [1, 0, 3, 2]
     v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));     // quad_perm [2, 3, 0, 1]
     v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));    // row_half_mirror
+    if (LANES == 16)                                                                                                // and the row of 16's mirror image
+        v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
     return v;
 }
 
-template <int R, bool PER_CHANNEL>
+template <int R, int LPC, bool PER_CHANNEL>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int ld, int q_col, int k_col, int v_col,
                                                          const float* __restrict__ beta, const float* __restrict__ decay,
                                                          float* __restrict__ state, const int* __restrict__ q_start,
                                                          const int* __restrict__ slots, float* __restrict__ o, int heads,
                                                          int kv_heads, int dim, int vdim) {
-    constexpr int DP = 8 * R;                               // a row's k (q, decay) padded with zeros to this many
+    constexpr int DP = LPC * R;                             // a row's k (q, decay) padded with zeros to this many
+    constexpr int kDeltaCols = 256 / LPC;                   // columns of the state a workgroup owns
     constexpr int NV = PER_CHANNEL ? 3 : 2;
     constexpr int W = NV * DP + kDeltaCols + 4;             // floats of a row in LDS: k, q, (decay,) v, beta, the head's decay
     constexpr int BLOCK = kDeltaRows * W;
@@ -307,7 +312,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     __shared__ float lds[2 * BLOCK];
     const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kDeltaCols;
     const int tid = threadIdx.x;
-    const int cl = tid / 8, l = tid % 8;
+    const int cl = tid / LPC, l = tid % LPC;
     const int col = col0 + cl;
     const bool live = col < vdim;
     const int kvh = h / (heads / kv_heads);
@@ -417,7 +422,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 m[i] *= PER_CHANNEL ? gg[i] : g_head;
                 dots[i % 2] += m[i] * kk[i];
             }
-            const float dot = sum_of_8_lanes(dots[0] + dots[1]);
+            const float dot = sum_of_lanes<LPC>(dots[0] + dots[1]);
             const float w = bt * (vv - dot);
             float reads[2] = {0.f, 0.f};
 #pragma unroll
@@ -425,7 +430,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
                 m[i] += kk[i] * w;
                 reads[i % 2] += m[i] * qq[i];
             }
-            const float read = sum_of_8_lanes(reads[0] + reads[1]);
+            const float read = sum_of_lanes<LPC>(reads[0] + reads[1]);
             if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read;
         }
         if (more) {
@@ -601,15 +606,16 @@ extern "C" int llme_delta_gates(const void* b_in, int ld_b, const void* a_in, in
     return launch_status();
 }
 
-template <int R>
-static void launch_delta_rule(bool per_channel, dim3 grid, hipStream_t stream, const float* qkv, int ld, int q_col, int k_col,
+template <int R, int LPC>
+static void launch_delta_rule(bool per_channel, int n_seq, hipStream_t stream, const float* qkv, int ld, int q_col, int k_col,
                               int v_col, const float* beta, const float* decay, float* state, const int* q_start,
                               const int* slots, float* o, int heads, int kv_heads, int dim, int vdim) {
+    const dim3 grid((vdim + 256 / LPC - 1) / (256 / LPC), heads, n_seq);
     if (per_channel)
-        delta_rule_kernel<R, true><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
+        delta_rule_kernel<R, LPC, true><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
                                                              heads, kv_heads, dim, vdim);
     else
-        delta_rule_kernel<R, false><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
+        delta_rule_kernel<R, LPC, false><<<grid, 256, 0, stream>>>(qkv, ld, q_col, k_col, v_col, beta, decay, state, q_start, slots, o,
                                                               heads, kv_heads, dim, vdim);
 }
 
@@ -621,17 +627,16 @@ extern "C" int llme_delta_rule(const void* qkv, int ld, int q_col, int k_col, in
     if (n_seq <= 0 || heads <= 0) return 0;
     if (kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return kErrBadArgument;
     if (dim > 256) return kErrUnsupported;
-    const dim3 grid((vdim + kDeltaCols - 1) / kDeltaCols, heads, n_seq);
-#define LLME_DELTA(R_)                                                                                                   \
-    launch_delta_rule<R_>(per_channel != 0, grid, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col,      \
+#define LLME_DELTA(R_, L_)                                                                                               \
+    launch_delta_rule<R_, L_>(per_channel != 0, n_seq, stream, static_cast<const float*>(qkv), ld, q_col, k_col, v_col, \
                           static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state), \
                           static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(o), heads, \
                           kv_heads, dim, vdim)
-    if (dim <= 16) LLME_DELTA(2);
-    else if (dim <= 32) LLME_DELTA(4);
-    else if (dim <= 64) LLME_DELTA(8);
-    else if (dim <= 128) LLME_DELTA(16);
-    else LLME_DELTA(32);
+    if (dim <= 16) LLME_DELTA(2, 8);
+    else if (dim <= 32) LLME_DELTA(4, 8);
+    else if (dim <= 64) LLME_DELTA(4, 16);
+    else if (dim <= 128) LLME_DELTA(8, 16);
+    else LLME_DELTA(16, 16);
 #undef LLME_DELTA
     return launch_status();
 }
