@@ -382,9 +382,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         const bool more = t0 + kDeltaRows < last;
         if (more) fetch(t0 + kDeltaRows);
         const int nt = min(kDeltaRows, last - t0);
-#pragma unroll
-        for (int tt = 0; tt < kDeltaRows; ++tt) {
-            if (tt >= nt) break;
+        auto one_row = [&](int tt) {
             const float* row = lds + cur * BLOCK + tt * W;
             const float vv = row[NV * DP + cl];
             const float bt = row[NV * DP + kDeltaCols];
@@ -432,6 +430,12 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
             }
             const float read = sum_of_lanes<LPC>(reads[0] + reads[1]);
             if (live && l == 0) o[static_cast<size_t>(t0 + tt) * heads * vdim + h * vdim + col] = read;
+        };
+        if (nt == kDeltaRows) {             // a whole block: no test between its rows, so that the rows' loads from LDS run ahead
+#pragma unroll
+            for (int tt = 0; tt < kDeltaRows; ++tt) one_row(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) one_row(tt);
         }
         if (more) {
             put(cur ^ 1);

@@ -139,6 +139,127 @@ __global__ __launch_bounds__(256) void sigmoid_attention_kernel(const TQ* __rest
     }
 }
 
+// Eight neighbouring values of a row of keys, queries or values, widened to 32-bit, in one or two loads.
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16>(const bf16* p, float (&v)[8]) {
+    typedef __attribute__((ext_vector_type(8))) __bf16 v8;
+    const v8 x = *reinterpret_cast<const v8*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<float>(x[i]);
+}
+
+// For rows that come one or a few to a request (decoding): one workgroup per (row, run of keys) as in the plain kernel,
+// but every thread reads whole lines. Per tile of 64 keys: (1) a thread takes a (key/value head, key) pair, reads the key's
+// row 16 bytes at a time and makes the scores of all query heads of that group against q in LDS; (2) a thread mixes the
+// heads' scores of eight (head, key) pairs and makes the weights; (3) a thread takes a (key/value head, value channel)
+// pair, reads its 64 tokens (contiguous in a page) and adds the group's heads' weighted values. dim and the page size are
+// multiples of 8, a group has at most PER query heads, G * 64 <= 256 NP and G * vdim <= 256 NP.
+template <typename TQ, typename TC, int PER, int NP>
+__global__ __launch_bounds__(256) void sigmoid_attention_rows_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
+                                                                     const TC* __restrict__ v_cache, const float* __restrict__ mix,
+                                                                     const float* __restrict__ bias, const int* __restrict__ positions,
+                                                                     const int* __restrict__ seq_idx, const int* __restrict__ block_table,
+                                                                     int max_blocks, float* __restrict__ partial, int T, int H, int G,
+                                                                     int dim, int vdim, int page, float scale, int run_len) {
+    extern __shared__ float lds[];
+    constexpr int KT = 64;
+    float* qs = lds;                    // [H][dim]
+    float* ms = qs + H * dim;           // [H][H]
+    float* bs = ms + H * H;             // [H]
+    float* sc = bs + H;                 // [H][KT + 1]
+    float* wt = sc + H * (KT + 1);      // [H][KT]
+    const int t = blockIdx.x, run = blockIdx.y, tid = threadIdx.x;
+    const int pos = positions[t];
+    const int key0 = run * run_len, key1 = min(pos + 1, key0 + run_len);
+    const int per = H / G;
+    float acc[NP][PER];
+#pragma unroll
+    for (int i = 0; i < NP; ++i)
+#pragma unroll
+        for (int u = 0; u < PER; ++u) acc[i][u] = 0.f;
+    if (key0 < key1) {
+        const int* table = block_table + static_cast<size_t>(seq_idx[t]) * max_blocks;
+        for (int e = tid; e < H * dim; e += 256) qs[e] = to_float(q[static_cast<size_t>(t) * H * dim + e]);
+        for (int e = tid; e < H * H; e += 256) ms[e] = mix[e];
+        for (int e = tid; e < H; e += 256) bs[e] = bias[e];
+        __syncthreads();
+        for (int j0 = key0; j0 < key1; j0 += KT) {
+            const int nk = min(KT, key1 - j0);
+            // (1) scores: pair = (kv, key)
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                const int pair = tid + 256 * i;
+                const int kv = pair / KT, j = pair % KT;
+                if (kv >= G) break;
+                float s[PER];
+#pragma unroll
+                for (int u = 0; u < PER; ++u) s[u] = 0.f;
+                if (j < nk) {
+                    const int key = j0 + j;
+                    const TC* kp = k_cache + ((static_cast<size_t>(table[key / page]) * G + kv) * page + key % page) * dim;
+                    for (int d = 0; d < dim; d += 8) {
+                        float kk[8];
+                        load8<TC>(kp + d, kk);
+#pragma unroll
+                        for (int u = 0; u < PER; ++u) {
+                            if (u >= per) break;
+                            const float* qp = qs + (kv * per + u) * dim + d;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) s[u] += qp[e] * kk[e];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < PER; ++u)
+                    if (u < per) sc[(kv * per + u) * (KT + 1) + j] = s[u] * scale;
+            }
+            __syncthreads();
+            // (2) mixed over the heads, then the weight
+            for (int e = tid; e < H * KT; e += 256) {
+                const int h = e / KT, j = e % KT;
+                float m = 0.f;
+                for (int g = 0; g < H; ++g) m += ms[h * H + g] * sc[g * (KT + 1) + j];
+                wt[e] = j < nk ? 1.0f / (1.0f + expf(-(m + bs[h]))) : 0.f;
+            }
+            __syncthreads();
+            // (3) weighted values: pair = (kv, value channel), the tile's keys eight at a time
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                const int pair = tid + 256 * i;
+                const int kv = pair / vdim, x = pair % vdim;
+                if (kv >= G) break;
+                for (int c = 0; c < nk; c += 8) {
+                    const int key = j0 + c;
+                    float vv[8];
+                    load8<TC>(v_cache + ((static_cast<size_t>(table[key / page]) * G + kv) * vdim + x) * page + key % page, vv);
+#pragma unroll
+                    for (int u = 0; u < PER; ++u) {
+                        if (u >= per) break;
+                        const float* wp = wt + (kv * per + u) * KT + c;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc[i][u] += wp[e] * vv[e];
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    float* out = partial + (static_cast<size_t>(run) * T + t) * H * vdim;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int pair = tid + 256 * i;
+        const int kv = pair / vdim, x = pair % vdim;
+        if (kv >= G) break;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (u < per) out[(kv * per + u) * vdim + x] = acc[i][u];
+    }
+}
+
 // The same on the matrix cores, for bfloat16 rows that come at least 16 to a request (prompts and their portions).
 // A workgroup owns 16 consecutive rows of one request and one run of its keys; each of its H / 4 wavefronts owns four
 // heads. Per tile of 32 keys: (1) every wavefront makes the transposed scores K Q^T of its heads (so that a lane holds,
@@ -346,10 +467,34 @@ static int launch_sigmoid_attention(const void* q, const void* k_cache, const vo
                                     const int* positions, const int* seq_idx, const int* block_table, int max_blocks,
                                     float* partial, int T, int H, int G, int dim, int vdim, int page, float scale, int run_len,
                                     int runs, hipStream_t stream) {
+    const dim3 grid(T, runs);
+    {
+        // the kernel that reads whole lines, where the sizes let it
+        const int per = H / G;
+        const int np = (G * (64 > vdim ? 64 : vdim) + 255) / 256;
+        const size_t lds_rows = sizeof(float) * (static_cast<size_t>(H) * dim + static_cast<size_t>(H) * H + H +
+                                                 static_cast<size_t>(H) * 65 + static_cast<size_t>(H) * 64);
+        if (dim % 8 == 0 && page % 8 == 0 && per <= 8 && np <= 4 && lds_rows <= 64 * 1024 &&
+            reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0) {
+#define LLME_SAR(P_, N_)                                                                                                 \
+    sigmoid_attention_rows_kernel<TQ, TC, P_, N_><<<grid, 256, lds_rows, stream>>>(                                      \
+        static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache), mix, bias, positions, \
+        seq_idx, block_table, max_blocks, partial, T, H, G, dim, vdim, page, scale, run_len)
+            const int pcode = per <= 1 ? 1 : per <= 2 ? 2 : per <= 4 ? 4 : 8;
+            const int ncode = np <= 1 ? 1 : np <= 2 ? 2 : 4;
+            switch (pcode * 10 + ncode) {
+                case 11: LLME_SAR(1, 1); break; case 12: LLME_SAR(1, 2); break; case 14: LLME_SAR(1, 4); break;
+                case 21: LLME_SAR(2, 1); break; case 22: LLME_SAR(2, 2); break; case 24: LLME_SAR(2, 4); break;
+                case 41: LLME_SAR(4, 1); break; case 42: LLME_SAR(4, 2); break; case 44: LLME_SAR(4, 4); break;
+                case 81: LLME_SAR(8, 1); break; case 82: LLME_SAR(8, 2); break; case 84: LLME_SAR(8, 4); break;
+            }
+#undef LLME_SAR
+            return launch_status();
+        }
+    }
     const size_t lds = sizeof(float) * (static_cast<size_t>(H) * dim + static_cast<size_t>(H) * H + H + 2 * static_cast<size_t>(H) * kKeysPerTile);
     if (lds > 64 * 1024) return kErrUnsupported;
     const int outs = H * vdim;
-    const dim3 grid(T, runs);
 #define LLME_SA(N_)                                                                                                      \
     sigmoid_attention_kernel<TQ, TC, N_><<<grid, 256, lds, stream>>>(                                                    \
         static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache), mix, bias, positions, \

@@ -318,6 +318,10 @@ def sigmoid_attention_mfma_fits(q: torch.Tensor, heads: int, dim: int, vdim: int
             and vdim % 16 == 0 and vdim <= 128 and page % 16 == 0)
 
 
+SIGMOID_ATTENTION_MFMA_ROWS = 4         # the most rows any request brings must reach this for the matrix-core kernel: a tile of
+                                        # 16 rows holding one does the mixing over heads 16 times over on the vector units
+
+
 def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, mix: torch.Tensor, bias: torch.Tensor,
                       gate: torch.Tensor, step, block_table: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                       dim: int, vdim: int, scale: float, scale_out: float = 1.0, mix_t: torch.Tensor | None = None) -> None:
@@ -343,11 +347,11 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         longest = max(c + n for c, n in zip(step.ctx_lens, step.new_lens))
     from .mfma import compute_units
     from .choices import choices_of
-    if (mix_t is not None and choices_of(step).fast_attention and sigmoid_attention_mfma_fits(q, heads, dim, vdim, page)):
-        # up to 16 rows of a request to a workgroup, scores and the second product on the matrix cores; single decoded
-        # tokens too (a tile of one row wastes matrix work, which is cheap; what counts there is that the keys are read
-        # in whole lines and cut into enough runs to fill the chip). The grid follows the step's shape only (a recorded
-        # step plans for the longest request its block tables hold).
+    if (mix_t is not None and choices_of(step).fast_attention and max(step.new_lens) >= SIGMOID_ATTENTION_MFMA_ROWS
+            and sigmoid_attention_mfma_fits(q, heads, dim, vdim, page)):
+        # a request brings several rows (prompts, portions; single tokens of other requests beside them ride along): up to
+        # 16 rows of a request to a workgroup, scores and the second product on the matrix cores. The grid follows the
+        # step's shape only.
         require(mix_t, "mix_t", torch.float32, (heads, heads))
         tiles = sum((n + 15) // 16 for n in step.new_lens)
         shortest_run = 256 if tiles >= 32 else 64
@@ -362,7 +366,8 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         check(entry("llme_sigmoid_attention_finish")(ptr(partial), runs, ptr(gate), ld_gate, ptr(out), code(out.dtype), ld_out, T,
                                                      heads, vdim, float(scale_out), stream()), "sigmoid_attention_finish")
         return
-    runs = max(1, min(64, (2 * compute_units()) // max(T, 1), (longest + 255) // 256))
+    # steps of single tokens: the kernel for few rows, the keys cut into runs of at least 64 until the chip is full
+    runs = max(1, min(64, -(-4 * compute_units() // max(T, 1)), (longest + 63) // 64))
     run_len = (longest + runs - 1) // runs
     run_len = (run_len + 31) // 32 * 32
     runs = max(1, (longest + run_len - 1) // run_len)

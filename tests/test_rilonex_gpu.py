@@ -65,6 +65,7 @@ ONE_LAYER = {
     "parallel": rm.config([rm.parallel(ff=None)], streams=None),
     "parallel_no_rotation_left_only": rm.config([rm.parallel(rot_dims=0, right_scale=0.0, ff=None)], streams=None),
     "parallel_right_only": rm.config([rm.parallel(left_scale=0.0, ff=None)], streams=None),
+    "parallel_key_size_of_20": rm.config([rm.parallel(heads=3, kv_heads=3, dim=20, vdim=12, rot_dims=10, ff=None)], streams=None),
     "feed_forward_and_streams": rm.config([rm.rglru(width=16, blocks=2, ff=56)], streams=4),
     "one_stream": rm.config([rm.channel_delta(ff=32)], streams=1),
     "one_tap_and_wide_keys": rm.config([rm.channel_delta(heads=2, kv_heads=1, dim=136, vdim=8, conv=1, ff=None),
