@@ -131,6 +131,74 @@ __global__ __launch_bounds__(256) void streams_read_norm_vec_kernel(const float*
     }
 }
 
+// write and the next sublayer's read_norm in one pass over a row: the new streams are stored and, still in registers,
+// mixed by the next sublayer's weights a2 and normed by w2 into out. Same limits as the vector form of read_norm.
+template <typename TW, typename TO, int NV4>
+__global__ __launch_bounds__(256) void streams_write_read_norm_kernel(float* __restrict__ x, int S, size_t stream_stride,
+                                                                      const float* __restrict__ mix, const float* __restrict__ b,
+                                                                      const float* __restrict__ y, const float* __restrict__ a2,
+                                                                      const TW* __restrict__ w2, TO* __restrict__ out, int H, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    float* xr = x + static_cast<size_t>(r) * H;
+    const float* yr = y + static_cast<size_t>(r) * H;
+    float m[kVecStreams][kVecStreams], bo[kVecStreams], coef[kVecStreams];
+#pragma unroll
+    for (int s = 0; s < kVecStreams; ++s) {
+        bo[s] = s < S ? b[s] : 0.f;
+        coef[s] = s < S ? a2[s] : 0.f;
+#pragma unroll
+        for (int t = 0; t < kVecStreams; ++t) m[s][t] = (s < S && t < S) ? mix[s * S + t] : 0.f;
+    }
+    float4 v[NV4][kVecStreams], yv[NV4];
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        const int i = (threadIdx.x + j * 256) * 4;
+        yv[j] = i < H ? *reinterpret_cast<const float4*>(yr + i) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < kVecStreams; ++s)
+            v[j][s] = (i < H && s < S) ? *reinterpret_cast<const float4*>(xr + static_cast<size_t>(s) * stream_stride + i)
+                                       : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float u[NV4][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        const int i = (threadIdx.x + j * 256) * 4;
+        u[j][0] = u[j][1] = u[j][2] = u[j][3] = 0.f;
+#pragma unroll
+        for (int t = 0; t < kVecStreams; ++t) {
+            if (t >= S) break;
+            float n[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < kVecStreams; ++s) {
+                n[0] += m[s][t] * v[j][s].x;
+                n[1] += m[s][t] * v[j][s].y;
+                n[2] += m[s][t] * v[j][s].z;
+                n[3] += m[s][t] * v[j][s].w;
+            }
+            n[0] += bo[t] * yv[j].x;
+            n[1] += bo[t] * yv[j].y;
+            n[2] += bo[t] * yv[j].z;
+            n[3] += bo[t] * yv[j].w;
+            if (i < H) *reinterpret_cast<float4*>(xr + static_cast<size_t>(t) * stream_stride + i) = float4{n[0], n[1], n[2], n[3]};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) u[j][e] += coef[t] * n[e];
+        }
+        ss += u[j][0] * u[j][0] + u[j][1] * u[j][1] + u[j][2] * u[j][2] + u[j][3] * u[j][3];
+    }
+    ss = block_sum(ss, scratch, 4);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+    TO* o = out + static_cast<size_t>(r) * H;
+#pragma unroll
+    for (int j = 0; j < NV4; ++j) {
+        const int i = (threadIdx.x + j * 256) * 4;
+        if (i >= H) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[i + e] = from_float<TO>((to_float(w2[i + e]) * u[j][e]) * inv);
+    }
+}
+
 __global__ __launch_bounds__(256) void streams_write_kernel(float* __restrict__ x, int S, size_t n, const float* __restrict__ mix,
                                                             const float* __restrict__ b, const float* __restrict__ y) {
     __shared__ float m[kMaxStreams * kMaxStreams];
@@ -207,6 +275,33 @@ extern "C" int llme_streams_read_norm(const void* x, int S, int T, int H, const 
         case 3: return launch_read_norm<bf16, bf16>(xp, S, stride, ap, w, out, rp, R, H, eps, stream);
     }
     return kErrBadArgument;
+}
+
+// write, then read_norm with the weights of the sublayer behind (a2 [S], w2 [H]) into out [T, H]: one kernel where the
+// vector form fits (returns kErrUnsupported otherwise, having done nothing: the caller then launches the two).
+extern "C" int llme_streams_write_read_norm(void* x, int S, int T, int H, const void* mix, const void* b, const void* y,
+                                            const void* a2, const void* w2, int w_dtype, void* out, int out_dtype, float eps,
+                                            hipStream_t stream) {
+    if (T <= 0 || H <= 0) return 0;
+    if (S < 1 || S > kVecStreams || H % 4 || H > 4096 || reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(y) % 16)
+        return kErrUnsupported;
+    const size_t stride = static_cast<size_t>(T) * H;
+#define LLME_SWR(TW_, TO_, N_)                                                                                            \
+    streams_write_read_norm_kernel<TW_, TO_, N_><<<T, 256, 0, stream>>>(                                                  \
+        static_cast<float*>(x), S, stride, static_cast<const float*>(mix), static_cast<const float*>(b),                  \
+        static_cast<const float*>(y), static_cast<const float*>(a2), static_cast<const TW_*>(w2), static_cast<TO_*>(out), H, eps)
+#define LLME_SWR_N(TW_, TO_)                                                                                              \
+    if (H <= 1024) LLME_SWR(TW_, TO_, 1); else if (H <= 2048) LLME_SWR(TW_, TO_, 2); else LLME_SWR(TW_, TO_, 4)
+    switch (w_dtype * 2 + out_dtype) {
+        case 0: LLME_SWR_N(float, float); break;
+        case 1: LLME_SWR_N(float, bf16); break;
+        case 2: LLME_SWR_N(bf16, float); break;
+        case 3: LLME_SWR_N(bf16, bf16); break;
+        default: return kErrBadArgument;
+    }
+#undef LLME_SWR_N
+#undef LLME_SWR
+    return launch_status();
 }
 
 // x [S, T, H] in place; mix [S, S] (from, to), b [S], y [T, H], all 32-bit.

@@ -117,8 +117,13 @@ class DecoderModel(Part):
         else:
             h = step.buffer("model.hidden", (T, self.hidden_size), torch.float32)
             self.embedding.forward(step.tokens, h, step)
-        for call in self.schedule:
-            self.layers[call.layer].forward(h, step, caches[call.cache_id], call.write_cache)
+        for i, call in enumerate(self.schedule):
+            layer = self.layers[call.layer]
+            if hasattr(layer, "next_block"):
+                # (a block that can hand the streams' next read on is told which layer runs behind it in this pass)
+                layer.next_block = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+            layer.forward(h, step, caches[call.cache_id], call.write_cache)
+        step.extra.pop("block.normed is for", None)
         if logit_rows is None or logit_rows.shape[0] == 0:
             return None
         R = logit_rows.shape[0]

@@ -25,6 +25,7 @@ GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
 declare("llme_streams_spread", [_vp, _i, _z, _vp])
 declare("llme_streams_read_norm", [_vp, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _f, _vp])
 declare("llme_streams_write", [_vp, _i, _z, _vp, _vp, _vp, _vp])
+declare("llme_streams_write_read_norm", [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _f, _vp])
 declare("llme_gated_act", [_vp, _i, _vp, _i, _i, _i, _i, _i, _vp])
 declare("llme_short_conv", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_rglru_gates", [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp])
@@ -100,6 +101,27 @@ def streams_write(x: torch.Tensor, mix: torch.Tensor, coef: torch.Tensor, y: tor
     require(coef, "coef", torch.float32, (S,))
     require(y, "y", torch.float32, (T, H))
     check(entry("llme_streams_write")(ptr(x), S, T * H, ptr(mix), ptr(coef), ptr(y), stream()), "streams_write")
+
+
+def streams_write_read_norm(x: torch.Tensor, mix: torch.Tensor, coef: torch.Tensor, y: torch.Tensor, next_coef: torch.Tensor,
+                            weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """streams_write(x, mix, coef, y) and then streams_read_norm(x, next_coef, weight, eps, out), as one kernel where the
+    sizes let it (up to 4 streams, rows of a multiple of 4 up to 4,096 values), else as the two."""
+    require(x, "x", torch.float32, (None, None, None))
+    S, T, H = x.shape
+    require(mix, "mix", torch.float32, (S, S))
+    require(coef, "coef", torch.float32, (S,))
+    require(next_coef, "next_coef", torch.float32, (S,))
+    require(y, "y", torch.float32, (T, H))
+    require(weight, "weight", _FLOATS, (H,))
+    require(out, "out", _FLOATS, (T, H))
+    status = entry("llme_streams_write_read_norm")(ptr(x), S, T, H, ptr(mix), ptr(coef), ptr(y), ptr(next_coef), ptr(weight),
+                                                   code(weight.dtype), ptr(out), code(out.dtype), float(eps), stream())
+    if status == 10002:
+        streams_write(x, mix, coef, y)
+        streams_read_norm(x, next_coef, weight, eps, out)
+        return
+    check(status, "streams_write_read_norm")
 
 
 # --- gated feed-forward activation -------------------------------------------------------

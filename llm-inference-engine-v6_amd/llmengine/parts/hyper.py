@@ -33,6 +33,9 @@ class HyperConnectionBlock(Block):
         if names:
             self.names.update(names)
         self.coef: dict = {}
+        # the block that runs behind this one when the model runs its layers in order (set by whoever composes the model;
+        # None: unknown, the blocks then do not hand their inputs on)
+        self.next_block = None
 
     def _subs(self):
         n = self.names
@@ -60,24 +63,52 @@ class HyperConnectionBlock(Block):
         for prefix, _, _ in self._subs():
             self.coef[prefix] = tuple(placement.place(get(f"{prefix}.{k}"), torch.float32) for k in ("in", "out", "mix"))
 
+    def first_read(self):
+        """(stream weights, norm weight, eps) of this block's first sublayer where its norm is the plain RMS formula, so that
+        the block in front can make this block's first input in the kernel that stores its own last result; else None."""
+        rms = self.mixer_norm.fused_rms()
+        return None if rms is None else (self.coef[self.names["mixer_streams"]][0], rms[0], rms[1])
+
     def forward(self, h, step, cache, write_cache=True):
         S, T, H = h.shape
         x = step.buffer("block.normed", (T, H), step.act_dtype)
         y = step.buffer("block.sublayer", (T, H), torch.float32)
-        for prefix, norm, sub in self._subs():
+        subs = self._subs()
+        # the block in front may have left this block's first input in x (see below)
+        ready = step.extra.pop("block.normed is for", None) == id(self)
+        for k, (prefix, norm, sub) in enumerate(subs):
             c_in, c_out, c_mix = self.coef[prefix]
-            rms = norm.fused_rms()
-            if rms is not None:
-                ops.streams_read_norm(h, c_in, rms[0], rms[1], x)
-            else:
-                u = step.buffer("block.mixed", (T, H), torch.float32)
-                ops.streams_read_norm(h, c_in, None, 0.0, u)
-                norm.forward(u, x)
+            if not ready:
+                rms = norm.fused_rms()
+                if rms is not None:
+                    ops.streams_read_norm(h, c_in, rms[0], rms[1], x)
+                else:
+                    u = step.buffer("block.mixed", (T, H), torch.float32)
+                    ops.streams_read_norm(h, c_in, None, 0.0, u)
+                    norm.forward(u, x)
+            ready = False
             if sub is self.mixer:
                 sub.forward(x, step, cache, y, False, write_cache)
             else:
                 sub.forward(x, step, y, False)
-            ops.streams_write(h, c_mix, c_out, y)
+            # what reads the streams next: this block's next sublayer, or the first sublayer of the block behind
+            if k + 1 < len(subs):
+                nxt_rms = subs[k + 1][1].fused_rms()
+                nxt = None if nxt_rms is None else (self.coef[subs[k + 1][0]][0], nxt_rms[0], nxt_rms[1])
+                owner = None
+            else:
+                behind = self.next_block
+                nxt = behind.first_read() if isinstance(behind, HyperConnectionBlock) and behind.streams == S else None
+                owner = behind
+            if nxt is not None:
+                # the streams' update and the next read of them in one pass over the rows
+                ops.streams_write_read_norm(h, c_mix, c_out, y, nxt[0], nxt[1], nxt[2], x)
+                if owner is not None:
+                    step.extra["block.normed is for"] = id(owner)
+                else:
+                    ready = True
+            else:
+                ops.streams_write(h, c_mix, c_out, y)
 
 
 register_part("block", "hyper", HyperConnectionBlock)
