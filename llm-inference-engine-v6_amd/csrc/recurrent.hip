@@ -44,6 +44,39 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
     out[static_cast<size_t>(t) * ld_out + c] = act == 1 ? siluf_(acc) : acc;
 }
 
+// A step in which every request brings one row (decoding): the convolution and the tail's move in one kernel. A thread
+// reads its channel's tail, makes the row's output and stores the tail moved on by the row.
+__global__ __launch_bounds__(256) void short_conv_single_kernel(const float* __restrict__ in, int ld_in, const float* __restrict__ w,
+                                                                const float* __restrict__ bias, const float* __restrict__ in_bias,
+                                                                float* __restrict__ tail, const int* __restrict__ seq_idx,
+                                                                const int* __restrict__ slots, float* __restrict__ out, int ld_out,
+                                                                int C, int K, int act) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float* tl = tail + static_cast<size_t>(slots[seq_idx[t]]) * (K - 1) * C;
+    const float x = in[static_cast<size_t>(t) * ld_in + c] + (in_bias ? in_bias[c] : 0.f);
+    float keep[kMaxTaps];
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+        if (i >= K - 1) break;
+        keep[i] = tl[static_cast<size_t>(i) * C + c];
+    }
+    float acc = bias ? bias[c] : 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+        if (i >= K - 1) break;
+        acc += w[static_cast<size_t>(c) * K + i] * keep[i];
+    }
+    acc += w[static_cast<size_t>(c) * K + K - 1] * x;
+    out[static_cast<size_t>(t) * ld_out + c] = act == 1 ? siluf_(acc) : acc;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+        if (i >= K - 1) break;
+        tl[static_cast<size_t>(i) * C + c] = i + 1 < K - 1 ? keep[i + 1] : x;
+    }
+}
+
 // The slot's tail after the step: the last K - 1 inputs of the request, from this step's rows and, where the
 // step brought fewer, from the old tail.
 __global__ __launch_bounds__(256) void conv_tail_kernel(const float* __restrict__ in, int ld_in,
@@ -501,6 +534,13 @@ extern "C" int llme_short_conv(const void* in, int ld_in, const void* w, const v
     if (T <= 0 || C <= 0) return 0;
     if (K < 1 || K > kMaxTaps) return kErrUnsupported;
     const dim3 grid((C + 255) / 256, T);
+    if (update_tail && T == n_seq) {            // one row per request
+        short_conv_single_kernel<<<grid, 256, 0, stream>>>(
+            static_cast<const float*>(in), ld_in, static_cast<const float*>(w), static_cast<const float*>(bias),
+            static_cast<const float*>(in_bias), static_cast<float*>(tail), static_cast<const int*>(seq_idx),
+            static_cast<const int*>(slots), static_cast<float*>(out), ld_out, C, K, act);
+        return launch_status();
+    }
     short_conv_kernel<<<grid, 256, 0, stream>>>(
         static_cast<const float*>(in), ld_in, static_cast<const float*>(w), static_cast<const float*>(bias),
         static_cast<const float*>(in_bias), static_cast<const float*>(tail), static_cast<const int*>(seq_idx), static_cast<const int*>(q_start),

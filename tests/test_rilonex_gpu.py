@@ -68,6 +68,7 @@ ONE_LAYER = {
     "parallel_key_size_of_20": rm.config([rm.parallel(heads=3, kv_heads=3, dim=20, vdim=12, rot_dims=10, ff=None)], streams=None),
     "feed_forward_and_streams": rm.config([rm.rglru(width=16, blocks=2, ff=56)], streams=4),
     "one_stream": rm.config([rm.channel_delta(ff=32)], streams=1),
+    "five_streams": rm.config([rm.rglru(width=16, blocks=1, ff=24), rm.channel_delta(ff=24)], streams=5),
     "one_tap_and_wide_keys": rm.config([rm.channel_delta(heads=2, kv_heads=1, dim=136, vdim=8, conv=1, ff=None),
                                         rm.rglru(width=24, blocks=2, conv=1, ff=None)], streams=None),
 }
