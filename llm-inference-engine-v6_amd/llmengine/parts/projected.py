@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from .. import ops
-from .base import CacheSpec, Getter, LayerCache, Mixer, ParamSpec, Placement
+from .base import CacheSpec, Getter, LayerCache, Mixer, Placement
 from .registry import register_part
 
 

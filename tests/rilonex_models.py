@@ -54,7 +54,6 @@ PLAIN = config([channel_delta(ff=None), rglru()], width=24, vocab=50, streams=No
 def make_weights(cfg: dict, seed: int, dtype=torch.bfloat16) -> dict:
     """name -> tensor for every tensor of the configuration's model (names and shapes as the engine's model
     tree lists them; the values are the tests' own)."""
-    import sys
     from llmengine.config.registry import architecture_name, parse_config, resolve
     model = resolve(architecture_name(cfg)).build_model(parse_config(cfg))
     g = torch.Generator().manual_seed(seed)

@@ -321,6 +321,38 @@ def test_the_models_trace_runner_replays_a_random_model(tmp_path):
             done[e["id"]] += len(e["tokens"])
 
 
+def test_the_command_line_generates_with_a_model_of_this_design(tmp_path):
+    """bin/llmengine-cli: greedy tokens of a model folder as the plain model chooses them, and sampling from a configuration
+    with random weights (which goes through the framework's own random initial values for this design's tensors)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg = rm.MIXED
+    folder, weights = rm.write_model(tmp_path / "model", cfg, 19, torch.float32)
+    prompt = _tokens(11, cfg["vocab"], 1)
+    want = list(prompt)
+    for _ in range(5):
+        want.append(int(plain.forward(cfg, weights, want)[0][-1].argmax()))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "llmengine-cli"), "--model", folder, "--dtype", "fp32",
+                          "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rec["token_ids"] == want and rec["finish_reason"] == "length"
+    cfgf = tmp_path / "cfg.json"
+    cfgf.write_text(json.dumps(rm.ALIGNED))
+    pf = tmp_path / "prompts.txt"
+    pf.write_text("1 2 3\n7,8,9,10,11\n")
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "llmengine-cli"), "--random", str(cfgf), "--seed", "3",
+                          "--prompt-file", str(pf), "--max-new-tokens", "4", "--temperature", "0.7"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    recs = [json.loads(line) for line in out.stdout.strip().splitlines()]
+    assert [len(r["token_ids"]) for r in recs] == [7, 9] and all(r["finish_reason"] == "length" for r in recs)
+
+
 def test_weights_with_a_rank_that_only_the_file_names(tmp_path):
     """The two-stage maps' inner sizes are read off the tensors when the configuration does not name them."""
     layer = rm.channel_delta(ff=None)
