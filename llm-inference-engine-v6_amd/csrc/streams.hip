@@ -19,6 +19,14 @@ __global__ __launch_bounds__(256) void streams_spread_kernel(float4* __restrict_
     }
 }
 
+// (value by value, for sizes that are no multiple of 4)
+__global__ __launch_bounds__(256) void streams_spread_scalar_kernel(float* __restrict__ x, int S, size_t n) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * 256) {
+        const float v = x[i];
+        for (int s = 1; s < S; ++s) x[static_cast<size_t>(s) * n + i] = v;
+    }
+}
+
 // One workgroup per output row. The row's mixed value is kept in registers between the two passes
 // (up to NV values per thread), or recomputed when the row is wider than that.
 template <typename TW, typename TO, int NV>
@@ -247,7 +255,11 @@ using namespace llme;
 
 extern "C" int llme_streams_spread(void* x, int S, size_t per_stream, hipStream_t stream) {
     if (S <= 1 || per_stream == 0) return 0;
-    if (per_stream % 4 || reinterpret_cast<uintptr_t>(x) % 16) return kErrBadArgument;
+    if (per_stream % 4 || reinterpret_cast<uintptr_t>(x) % 16) {
+        const int blocks = static_cast<int>(per_stream / 256 + 1 < 4096 ? per_stream / 256 + 1 : 4096);
+        streams_spread_scalar_kernel<<<blocks, 256, 0, stream>>>(static_cast<float*>(x), S, per_stream);
+        return launch_status();
+    }
     const size_t n4 = per_stream / 4;
     const int grid = static_cast<int>(n4 / 256 + 1 < 4096 ? n4 / 256 + 1 : 4096);
     streams_spread_kernel<<<grid, 256, 0, stream>>>(static_cast<float4*>(x), S, n4);

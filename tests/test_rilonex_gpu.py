@@ -68,6 +68,9 @@ ONE_LAYER = {
     "parallel_key_size_of_20": rm.config([rm.parallel(heads=3, kv_heads=3, dim=20, vdim=12, rot_dims=10, ff=None)], streams=None),
     "feed_forward_and_streams": rm.config([rm.rglru(width=16, blocks=2, ff=56)], streams=4),
     "one_stream": rm.config([rm.channel_delta(ff=32)], streams=1),
+    "width_of_30": rm.config([rm.rglru(width=18, blocks=3, ff=14), rm.parallel(heads=2, kv_heads=1, dim=6, vdim=10, rot_dims=4, d_heads=1,
+                                                                             d_kv=1, d_dim=6, d_vdim=10, ff=None)],
+                             width=30, vocab=33, streams=3),
     "five_streams": rm.config([rm.rglru(width=16, blocks=1, ff=24), rm.channel_delta(ff=24)], streams=5),
     "one_tap_and_wide_keys": rm.config([rm.channel_delta(heads=2, kv_heads=1, dim=136, vdim=8, conv=1, ff=None),
                                         rm.rglru(width=24, blocks=2, conv=1, ff=None)], streams=None),
@@ -85,6 +88,21 @@ def test_each_mechanism_alone_whole_and_token_by_token(tmp_path, name):
         got = replay.run_trace(engine, cache, steps)
         assert _covered(got, requests)
         assert _worst(got, ref) < F32_TOL
+
+
+@pytest.mark.parametrize("name", ["width_of_30", "parallel_key_size_of_20", "one_tap_and_wide_keys", "five_streams"])
+def test_sizes_that_no_fast_kernel_takes_in_bfloat16(tmp_path, name):
+    """Widths, key sizes and stream counts that fall outside the vector and matrix-core kernels' limits, served in bfloat16:
+    the plain kernels carry them, whole prompts and single tokens agree, and both are the plain model's within rounding."""
+    cfg = ONE_LAYER[name]
+    engine, weights = _engine(tmp_path, cfg, 4, "bf16")
+    requests = {"a": _tokens(45, cfg["vocab"], 1), "b": _tokens(3, cfg["vocab"], 2)}
+    ref = _reference(cfg, {k: v.float() for k, v in weights.items()}, requests)
+    whole = replay.run_trace(engine, engine.new_cache(8, 16, 2), replay.whole(requests))
+    tail = replay.run_trace(engine, engine.new_cache(8, 16, 2), replay.tail_one_by_one(requests, tail=40))
+    assert _covered(whole, requests) and _covered(tail, requests)
+    assert _mean(whole, ref) < BF16_MEAN and _worst(whole, ref) < BF16_WORST
+    assert _worst(tail, {rid: np.stack([whole[rid][p] for p in sorted(whole[rid])]) for rid in requests}) < BF16_BETWEEN_SCHEDULES
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
