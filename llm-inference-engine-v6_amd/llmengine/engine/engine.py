@@ -68,7 +68,8 @@ class BlockManager:
     def free_blocks(self) -> int:
         if self._cache is None:
             return self._num_blocks
-        return min(self._cache.manager.free_pages(g) for g in self._cache.manager.groups)
+        # (a model that keeps no pages, only states of fixed size, uses none of them)
+        return min((self._cache.manager.free_pages(g) for g in self._cache.manager.groups), default=self._num_blocks)
 
 
 class Engine:
@@ -304,7 +305,7 @@ class Engine:
         if c is not None:
             for r in c.manager.live_requests():
                 c.release(r)
-            if min(c.manager.num_pages(g) for g in c.manager.groups) >= pages:
+            if min((c.manager.num_pages(g) for g in c.manager.groups), default=pages) >= pages:
                 return c
             self._own_cache = c = None          # drop the small pool before making the larger one
         self._own_cache = self.new_cache(pages, self.block_size, 1)

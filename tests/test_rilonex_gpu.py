@@ -309,6 +309,40 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(tmp_path):
     assert [r.token_ids for r in sched.results] == want
 
 
+def test_a_model_without_pages_generates_again_and_again(tmp_path):
+    """Recurrent layers only: no mixer keeps pages, the engine's own pool and the scheduler's have nothing to count."""
+    cfg = rm.PLAIN
+    engine, weights = _engine(tmp_path, cfg, 20, "fp32")
+    prompt = _tokens(7, cfg["vocab"], 1)
+    want = list(prompt)
+    for _ in range(4):
+        want.append(int(plain.forward(cfg, weights, want)[0][-1].argmax()))
+    for _ in range(3):
+        assert engine.generate(prompt, 4)[0] == want
+    from llmengine import BlockManager, ContinuousBatchScheduler
+    blocks = BlockManager(num_blocks=4, block_size=16)
+    sched = ContinuousBatchScheduler(engine, blocks, max_concurrent=2, max_prefill_tokens_per_step=8)
+    for _ in range(3):
+        sched.enqueue(prompt, 4)
+    sched.run_until_idle()
+    assert [r.token_ids for r in sched.results] == [want] * 3 and blocks.free_blocks == 4
+
+
+@pytest.mark.parametrize("dtype", ["bf16"])
+def test_thirty_two_heads_on_the_matrix_cores(tmp_path, dtype):
+    """32 query heads: eight wavefronts a workgroup and more LDS than a kernel gets without asking."""
+    cfg = rm.config([rm.parallel(heads=32, kv_heads=8, dim=32, vdim=16, rot_dims=32, scale=0.4, right_scale=0.0, ff=None)],
+                    streams=None, width=64)
+    weights = _sharp_attention(cfg, rm.make_weights(cfg, 23, torch.bfloat16), far_scale=3.0)
+    engine, _ = _engine(tmp_path, cfg, 23, dtype, weights=weights)
+    requests = {"a": _tokens(200, cfg["vocab"], 1), "b": _tokens(21, cfg["vocab"], 2)}
+    ref = _reference(cfg, {k: v.float() for k, v in weights.items()}, requests)
+    whole = replay.run_trace(engine, engine.new_cache(16, 16, 2), replay.whole(requests))
+    tail = replay.run_trace(engine, engine.new_cache(16, 16, 2), replay.tail_one_by_one(requests, tail=20))
+    assert _mean(whole, ref) < BF16_MEAN and _worst(whole, ref) < BF16_WORST
+    assert _worst(tail, {rid: np.stack([whole[rid][p] for p in sorted(whole[rid])]) for rid in requests}) < 3e-3
+
+
 def test_the_models_trace_runner_replays_a_random_model(tmp_path):
     """bin/trace_run on a model folder of this design: mixed steps, four slots, logits as files."""
     import json
