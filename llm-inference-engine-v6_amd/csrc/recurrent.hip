@@ -543,8 +543,8 @@ extern "C" int llme_short_conv(const void* in, int ld_in, const void* w, const v
     }
     short_conv_kernel<<<grid, 256, 0, stream>>>(
         static_cast<const float*>(in), ld_in, static_cast<const float*>(w), static_cast<const float*>(bias),
-        static_cast<const float*>(in_bias), static_cast<const float*>(tail), static_cast<const int*>(seq_idx), static_cast<const int*>(q_start),
-        static_cast<const int*>(slots), static_cast<float*>(out), ld_out, C, K, act);
+        static_cast<const float*>(in_bias), static_cast<const float*>(tail), static_cast<const int*>(seq_idx),
+        static_cast<const int*>(q_start), static_cast<const int*>(slots), static_cast<float*>(out), ld_out, C, K, act);
     if (update_tail && K > 1)
         conv_tail_kernel<<<dim3((C + 255) / 256, n_seq), 256, 0, stream>>>(
             static_cast<const float*>(in), ld_in, static_cast<const float*>(in_bias), static_cast<float*>(tail),

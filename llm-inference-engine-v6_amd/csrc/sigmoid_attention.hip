@@ -456,6 +456,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_finish_kernel(const flo
     const size_t per_run = static_cast<size_t>(T) * H * vdim;
     for (int e = blockIdx.y * 256 + threadIdx.x; e < H * vdim; e += gridDim.y * 256) {
         float a = 0.f;
+#pragma unroll 8
         for (int r = 0; r < runs; ++r) a += partial[r * per_run + static_cast<size_t>(t) * H * vdim + e];
         const float g = 1.0f / (1.0f + expf(-gate[static_cast<size_t>(t) * ld_gate + e / vdim]));
         out[static_cast<size_t>(t) * ld_out + e] = from_float<TO>(scale_out * (g * a));
