@@ -1,0 +1,205 @@
+"""Python faces of the kernels for sandwich norms, latent attention and mixtures of experts. As everywhere
+in ops: operands are checked on the host, then the kernel is launched on the current stream; nothing
+computes on the host."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .lib import KernelError, check, code, declare, entry, ptr, require, stream
+
+_vp, _i, _f, _z, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_long
+_FLOATS = (torch.float32, torch.bfloat16)
+LATENT_MAX_ROW, LATENT_MAX_RANK = 1024, 512         # the plain attention kernel's limits (cached row, latent)
+MOE_MAX_EXPERTS = 1024
+MOE_TILE = 16
+
+declare("llme_norm_add", [_vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _f, _vp])
+declare("llme_scale_f32", [_vp, _z, _f, _vp])
+declare("llme_latent_prepare", [_vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp])
+declare("llme_latent_q_rotate", [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp])
+declare("llme_head_gemm", [_vp, _i, _l, _l, _vp, _i, _vp, _i, _l, _l, _i, _i, _i, _i, _vp])
+declare("llme_latent_attention", [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp])
+declare("llme_moe_route", [_vp, _i, _i, _i, _f, _i, _vp, _vp, _vp])
+declare("llme_moe_plan", [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp])
+declare("llme_moe_gemm", [_vp, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+declare("llme_moe_combine", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
+
+
+# --- sandwich norm ---------------------------------------------------------------------
+def norm_add(y: torch.Tensor, w_post: torch.Tensor, h: torch.Tensor, eps: float, w_next: torch.Tensor | None = None,
+             x_out: torch.Tensor | None = None) -> None:
+    """h += w_post * y / rms(y); with w_next also x_out = w_next * h / rms(h) of the updated rows.
+    y, h [T, H] 32-bit; the weights multiply as they are."""
+    require(y, "y", torch.float32, (None, None))
+    T, H = y.shape
+    require(h, "h", torch.float32, (T, H))
+    require(w_post, "w_post", _FLOATS, (H,))
+    if w_next is not None:
+        require(w_next, "w_next", w_post.dtype, (H,))
+        require(x_out, "x_out", _FLOATS, (T, H))
+    check(entry("llme_norm_add")(ptr(y), ptr(w_post), code(w_post.dtype), ptr(h), ptr(w_next),
+                                 code(w_next.dtype) if w_next is not None else 0, ptr(x_out) if w_next is not None else None,
+                                 code(x_out.dtype) if w_next is not None else 0, T, H, float(eps), stream()), "norm_add")
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    """x *= s, in place (32-bit)."""
+    require(x, "x", torch.float32)
+    check(entry("llme_scale_f32")(ptr(x), x.numel(), float(s), stream()), "scale")
+
+
+# --- latent attention ------------------------------------------------------------------
+def latent_prepare(p: torch.Tensor, q_rank: int, kv_rank: int, rot: int, rot_dims: int, wq: torch.Tensor, wc: torch.Tensor | None,
+                   freq: torch.Tensor | None, mag: float, step, block_table: torch.Tensor | None, cq: torch.Tensor,
+                   cache: torch.Tensor | None, eps: float) -> None:
+    """p [T, >= q_rank + kv_rank + rot] 32-bit (the down maps' outputs side by side) -> cq [T, q_rank], the
+    RMS-normed query latent, and the cache rows [normed latent | shared key part, its first rot_dims entries
+    rotated] at the tokens' places. kv_rank = 0: queries only (a layer that reads another layer's rows)."""
+    require(p, "p", torch.float32, (None, None))
+    T, ld = p.shape
+    if ld < q_rank + kv_rank + rot:
+        raise KernelError(f"latent_prepare: rows of {ld} hold no {q_rank} + {kv_rank} + {rot} columns")
+    require(wq, "wq", _FLOATS, (q_rank,))
+    require(cq, "cq", _FLOATS, (T, q_rank))
+    page = 0
+    if kv_rank:
+        require(wc, "wc", wq.dtype, (kv_rank,))
+        require(cache, "cache", cq.dtype, (None, None, kv_rank + rot))
+        require(block_table, "block_table", torch.int32, (None, None))
+        page = cache.shape[1]
+        if rot_dims:
+            require(freq, "freq", torch.float32, (rot_dims // 2,))
+    check(entry("llme_latent_prepare")(
+        ptr(p), ld, q_rank, kv_rank, rot if kv_rank else 0, rot_dims if kv_rank else 0, ptr(wq), ptr(wc) if kv_rank else None, code(wq.dtype),
+        ptr(freq) if (kv_rank and rot_dims) else None, float(mag), ptr(step.positions), ptr(step.seq_idx),
+        ptr(block_table) if kv_rank else None, block_table.shape[1] if kv_rank else 0, ptr(cq),
+        ptr(cache) if kv_rank else None, code(cq.dtype), page, T, float(eps), stream()), "latent_prepare")
+
+
+def latent_q_rotate(q: torch.Tensor, freq: torch.Tensor | None, mag: float, positions: torch.Tensor, qp: torch.Tensor,
+                    heads: int, dim: int, rot: int, rot_dims: int, kv_rank: int) -> None:
+    """The last `rot` entries of every head of q [T, heads (dim + rot)], the first rot_dims of them rotated,
+    into the last `rot` entries of every head of qp [T, heads (kv_rank + rot)]."""
+    T = q.shape[0]
+    require(q, "q", _FLOATS, (T, heads * (dim + rot)))
+    require(qp, "qp", q.dtype, (T, heads * (kv_rank + rot)))
+    if rot_dims:
+        require(freq, "freq", torch.float32, (rot_dims // 2,))
+    require(positions, "positions", torch.int32, (T,))
+    check(entry("llme_latent_q_rotate")(ptr(q), code(q.dtype), ptr(freq) if rot_dims else None, float(mag), ptr(positions),
+                                        ptr(qp), T, heads, dim, rot, rot_dims, kv_rank, stream()), "latent_q_rotate")
+
+
+_fast_head_gemm = None          # set by ops/latent_mfma.py
+
+
+def head_gemm(a: torch.Tensor, a_cols: int, w: torch.Tensor, out: torch.Tensor, out_cols: int, heads: int,
+              choices=None) -> None:
+    """out[t, h, :N] = w[h] a[t, h, :K] for w [heads, N, K]; a [T, heads * a_cols] and out [T, heads * out_cols]
+    hold a head's K inputs and N outputs at the start of its a_cols / out_cols columns."""
+    require(w, "w", _FLOATS, (heads, None, None))
+    _, N, K = w.shape
+    T = a.shape[0]
+    require(a, "a", _FLOATS, (T, heads * a_cols))
+    require(out, "out", a.dtype, (T, heads * out_cols))
+    if K > a_cols or N > out_cols:
+        raise KernelError(f"head_gemm: {K} inputs and {N} outputs do not fit heads of {a_cols} and {out_cols} columns")
+    if _fast_head_gemm is not None and _fast_head_gemm(a, a_cols, w, out, out_cols, heads, choices):
+        return
+    check(entry("llme_head_gemm")(ptr(a), code(a.dtype), heads * a_cols, a_cols, ptr(w), code(w.dtype), ptr(out),
+                                  code(out.dtype), heads * out_cols, out_cols, T, heads, N, K, stream()), "head_gemm")
+
+
+def latent_attention_fits(kv_rank: int, rot: int) -> bool:
+    return kv_rank <= LATENT_MAX_RANK and kv_rank + rot <= LATENT_MAX_ROW
+
+
+_fast_latent_attention = None   # set by ops/latent_mfma.py
+
+
+def latent_attention(qp: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, step, block_table: torch.Tensor,
+                     heads: int, kv_rank: int, scale: float, window: int = 0) -> None:
+    """out[t, h] = sum_j softmax_j(scale qp[t, h] . row_j) row_j[:kv_rank] over the rows of the token's request
+    that it may see (all up to its own; with a window the last `window` of them)."""
+    T = qp.shape[0]
+    require(cache, "cache", _FLOATS, (None, None, None))
+    D = cache.shape[2]
+    require(qp, "qp", cache.dtype, (T, heads * D))
+    require(out, "out", qp.dtype, (T, heads * kv_rank))
+    require(block_table, "block_table", torch.int32, (None, None))
+    if not latent_attention_fits(kv_rank, D - kv_rank):
+        raise KernelError(f"latent attention: rows of {D} with a latent of {kv_rank} are beyond the kernel's limits")
+    if _fast_latent_attention is not None and _fast_latent_attention(qp, cache, out, step, block_table, heads, kv_rank,
+                                                                     scale, window):
+        return
+    check(entry("llme_latent_attention")(ptr(qp), code(qp.dtype), ptr(cache), code(cache.dtype), ptr(out),
+                                         ptr(step.positions), ptr(step.seq_idx), ptr(block_table), block_table.shape[1],
+                                         T, heads, kv_rank, D, cache.shape[1], float(scale), int(window), stream()),
+          "latent_attention")
+
+
+# --- mixture of experts ----------------------------------------------------------------
+def moe_capacity(pairs: int, experts: int) -> int:
+    """Places for `pairs` (token, expert) pairs when every expert's run is padded to whole tiles."""
+    return (pairs + experts * (MOE_TILE - 1) + MOE_TILE - 1) // MOE_TILE * MOE_TILE
+
+
+def moe_route(logits: torch.Tensor, top: int, scale: float, renormalize: bool, ids: torch.Tensor, wts: torch.Tensor) -> None:
+    require(logits, "logits", torch.float32, (None, None))
+    T, E = logits.shape
+    require(ids, "ids", torch.int32, (T, top))
+    require(wts, "wts", torch.float32, (T, top))
+    check(entry("llme_moe_route")(ptr(logits), T, E, top, float(scale), 1 if renormalize else 0, ptr(ids), ptr(wts), stream()),
+          "moe_route")
+
+
+def moe_plan(ids: torch.Tensor, experts: int, place_pair: torch.Tensor, pair_place: torch.Tensor,
+             tile_expert: torch.Tensor, n_tiles: torch.Tensor) -> None:
+    require(ids, "ids", torch.int32, (None, None))
+    pairs = ids.numel()
+    cap = moe_capacity(pairs, experts)
+    require(place_pair, "place_pair", torch.int32, (cap,))
+    require(pair_place, "pair_place", torch.int32, (pairs,))
+    require(tile_expert, "tile_expert", torch.int32, (cap // MOE_TILE,))
+    require(n_tiles, "n_tiles", torch.int32, (1,))
+    check(entry("llme_moe_plan")(ptr(ids), pairs, experts, MOE_TILE, cap, ptr(place_pair), ptr(pair_place), ptr(tile_expert),
+                                 ptr(n_tiles), stream()), "moe_plan")
+
+
+_fast_moe_gemm = None           # set by ops/latent_mfma.py
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, w2: torch.Tensor | None, out: torch.Tensor, place_pair: torch.Tensor,
+             tile_expert: torch.Tensor, n_tiles: torch.Tensor, gather_div: int, activation: str = "silu", choices=None) -> None:
+    """Per place: out[place] = w[expert] a[row] (w2 given: act(w a) * (w2 a)); row = pair // gather_div, or the
+    place itself where gather_div is 0. w, w2 [experts, N, K]."""
+    from .recurrent import GATE_ACTIVATIONS
+    require(w, "w", _FLOATS, (None, None, None))
+    E, N, K = w.shape
+    if w2 is not None:
+        require(w2, "w2", w.dtype, (E, N, K))
+    require(a, "a", _FLOATS, (None, K))
+    cap = place_pair.shape[0]
+    require(out, "out", _FLOATS, (cap, N))
+    require(tile_expert, "tile_expert", torch.int32, (cap // MOE_TILE,))
+    if gather_div == 0 and a.shape[0] != cap:
+        raise KernelError("moe_gemm: rows by place need one row per place")
+    if _fast_moe_gemm is not None and _fast_moe_gemm(a, w, w2, out, place_pair, tile_expert, n_tiles, gather_div,
+                                                     activation, choices):
+        return
+    check(entry("llme_moe_gemm")(ptr(a), code(a.dtype), ptr(w), ptr(w2), code(w.dtype), ptr(out), code(out.dtype),
+                                 ptr(place_pair), ptr(tile_expert), ptr(n_tiles), cap // MOE_TILE, int(gather_div), N, K,
+                                 GATE_ACTIVATIONS[activation], stream()), "moe_gemm")
+
+
+def moe_combine(y: torch.Tensor, pair_place: torch.Tensor, wts: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+    require(out, "out", torch.float32, (None, None))
+    T, H = out.shape
+    require(wts, "wts", torch.float32, (T, None))
+    top = wts.shape[1]
+    require(y, "y", torch.float32, (None, H))
+    require(pair_place, "pair_place", torch.int32, (T * top,))
+    check(entry("llme_moe_combine")(ptr(y), ptr(pair_place), ptr(wts), ptr(out), T, top, H, 1 if accumulate else 0, stream()),
+          "moe_combine")

@@ -6,6 +6,9 @@ residual stream h is 32-bit; mixer and feed-forward add their result into it
 """
 from __future__ import annotations
 
+import torch
+
+from .. import ops
 from .base import Block, FeedForward, Mixer, Norm
 from .registry import register_part
 
@@ -47,4 +50,64 @@ class PreNormBlock(Block):
             self.feed_forward.forward(x, step, h, True)
 
 
+class SandwichBlock(Block):
+    """A norm in front of and behind every sublayer: h += post1(mixer(pre1(h))); h += post2(ffn(pre2(h))).
+    A sublayer's result is a 32-bit buffer of its own; the norm behind it, the sum into the stream and the
+    norm in front of whatever reads the stream next (this block's feed-forward, or the first sublayer of
+    the block behind) are one kernel where all three norms are the plain RMS formula."""
+    graph_safe = True
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm, ffn_norm: Norm | None,
+                 mixer_post_norm: Norm, ffn_post_norm: Norm | None, names: dict | None = None):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+        self.mixer_post_norm, self.ffn_post_norm = mixer_post_norm, ffn_post_norm
+        self.names = {"mixer_norm": "norm1", "mixer": "mix", "mixer_post_norm": "norm1b",
+                      "ffn_norm": "norm2", "feed_forward": "mlp", "ffn_post_norm": "norm2b"}
+        if names:
+            self.names.update(names)
+        # the block that runs behind this one (told by the model as it runs its schedule; None: unknown)
+        self.next_block = None
+
+    def children(self):
+        n = self.names
+        out = {n["mixer_norm"]: self.mixer_norm, n["mixer_post_norm"]: self.mixer_post_norm, n["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out.update({n["ffn_norm"]: self.ffn_norm, n["ffn_post_norm"]: self.ffn_post_norm,
+                        n["feed_forward"]: self.feed_forward})
+        return out
+
+    def _join(self, y, post: Norm, h, nxt: Norm | None, x, step) -> bool:
+        """h += post(y); True if x was also made = nxt(h)."""
+        rms = post.fused_rms()
+        nxt_rms = nxt.fused_rms() if nxt is not None else None
+        if rms is not None and nxt_rms is not None and nxt_rms[0].dtype == rms[0].dtype and nxt_rms[1] == rms[1]:
+            ops.norm_add(y, rms[0], h, rms[1], nxt_rms[0], x)
+            return True
+        if rms is not None:
+            ops.norm_add(y, rms[0], h, rms[1])
+        else:
+            raise NotImplementedError("sandwich blocks take norms of the plain RMS formula behind their sublayers")
+        return False
+
+    def forward(self, h, step, cache, write_cache=True):
+        T, H = h.shape
+        x = step.buffer("block.normed", (T, H), step.act_dtype)
+        y = step.buffer("block.sublayer", (T, H), torch.float32)
+        if step.extra.pop("block.normed is for", None) != id(self):
+            self.mixer_norm.forward(h, x)
+        self.mixer.forward(x, step, cache, y, False, write_cache)
+        behind = self.next_block.mixer_norm if isinstance(self.next_block, SandwichBlock) else None
+        if self.feed_forward is None:
+            if self._join(y, self.mixer_post_norm, h, behind, x, step):
+                step.extra["block.normed is for"] = id(self.next_block)
+            return
+        if not self._join(y, self.mixer_post_norm, h, self.ffn_norm, x, step):
+            self.ffn_norm.forward(h, x)
+        self.feed_forward.forward(x, step, y, False)
+        if self._join(y, self.ffn_post_norm, h, behind, x, step):
+            step.extra["block.normed is for"] = id(self.next_block)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

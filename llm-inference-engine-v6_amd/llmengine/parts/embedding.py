@@ -16,9 +16,10 @@ from .registry import register_part
 class Embedding(TokenEmbedding):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensor: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tensor: str = "weight", scale: float = 1.0):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tensor = tensor            # the local name of the table ("": the part's own name)
+        self.scale = float(scale)       # a multiplier on every row, applied in 32-bit
         self.weight: torch.Tensor | None = None
 
     def param_specs(self):
@@ -30,6 +31,8 @@ class Embedding(TokenEmbedding):
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor, step=None) -> None:
         ops.embed_gather(self.weight, tokens, out)
+        if self.scale != 1.0:
+            ops.scale_(out, self.scale)
 
 
 class OutputHead(Head):

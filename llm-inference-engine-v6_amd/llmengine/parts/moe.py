@@ -1,0 +1,83 @@
+"""Mixture of experts: a router scores E small gated feed-forward layers for every token, the token runs
+the `top` best of them, and their results are added with the router's weights; a shared expert of the same
+form may run for every token beside them.
+
+Router: z = Wr x in 32-bit (the matrix is kept in 32-bit), s = softmax(z) over all experts, the `top`
+largest s are chosen (the lower index wins a tie), weight = s * scale, divided by the chosen scores' sum
+first where `renormalize` is set. Expert e: down_e(act(gate_e x) * up_e x), no biases. Tensors: "router",
+"e<i>.gate", "e<i>.up", "e<i>.down"; the shared expert is a child part under "shared".
+
+On the device the (token, expert) pairs are grouped by expert into tiles of rows, and two grouped products
+(gate/up with the activation, then down) run over the tiles; nothing of the routing comes to the host, so
+a step's launches do not depend on what the tokens choose.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import FeedForward, Getter, ParamSpec, Placement
+from .registry import register_part
+
+
+class MixtureOfExperts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, scale: float = 1.0,
+                 renormalize: bool = False, activation: str = "silu", shared: FeedForward | None = None,
+                 expert_name: str = "e{}"):
+        if not 1 <= top <= experts:
+            raise ValueError(f"top={top} must be between 1 and experts={experts}")
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"mixture_of_experts: activation {activation!r} is none of {sorted(ops.GATE_ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.experts, self.top, self.scale = int(experts), int(top), float(scale)
+        self.renormalize, self.activation = bool(renormalize), activation
+        self.shared, self.expert_name = shared, expert_name
+
+    def children(self):
+        return {"shared": self.shared} if self.shared is not None else {}
+
+    def refusals(self):
+        if self.experts > ops.latent.MOE_MAX_EXPERTS:
+            return [f"experts={self.experts}: the routing kernels take up to {ops.latent.MOE_MAX_EXPERTS}"]
+        return []
+
+    def param_specs(self):
+        H, FF = self.hidden_size, self.intermediate_size
+        out = {"router": ParamSpec((self.experts, H))}
+        for e in range(self.experts):
+            name = self.expert_name.format(e)
+            out.update({f"{name}.gate": ParamSpec((FF, H)), f"{name}.up": ParamSpec((FF, H)), f"{name}.down": ParamSpec((H, FF))})
+        return out
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        self.w_router = placement.place(get("router"), torch.float32)
+        names = [self.expert_name.format(e) for e in range(self.experts)]
+        dtype = placement.common_dtype([get(f"{names[0]}.{k}") for k in ("gate", "up", "down")])
+        stack = lambda key: torch.stack([placement.place(get(f"{n}.{key}"), dtype) for n in names]).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+
+    def forward(self, x, step, out, accumulate):
+        T, H = x.shape
+        E, top, FF = self.experts, self.top, self.intermediate_size
+        i32, f32 = torch.int32, torch.float32
+        logits = step.buffer("moe.logits", (T, E), f32)
+        ops.gemm(x, self.w_router, logits, choices=step.choices)
+        ids, wts = step.buffer("moe.ids", (T, top), i32), step.buffer("moe.weights", (T, top), f32)
+        ops.moe_route(logits, top, self.scale, self.renormalize, ids, wts)
+        cap = ops.moe_capacity(T * top, E)
+        place_pair, pair_place = step.buffer("moe.place_pair", (cap,), i32), step.buffer("moe.pair_place", (T * top,), i32)
+        tile_expert, n_tiles = step.buffer("moe.tile_expert", (cap // ops.latent.MOE_TILE,), i32), step.buffer("moe.tiles", (1,), i32)
+        ops.moe_plan(ids, E, place_pair, pair_place, tile_expert, n_tiles)
+        act = step.buffer("moe.act", (cap, FF), step.act_dtype)
+        ops.moe_gemm(x, self.w_gate, self.w_up, act, place_pair, tile_expert, n_tiles, top, self.activation, step.choices)
+        y = step.buffer("moe.y", (cap, H), f32)
+        ops.moe_gemm(act, self.w_down, None, y, place_pair, tile_expert, n_tiles, 0, self.activation, step.choices)
+        if self.shared is not None:
+            self.shared.forward(x, step, out, accumulate)
+            accumulate = True
+        ops.moe_combine(y, pair_place, wts, out, accumulate)
+
+
+register_part("feed_forward", "mixture_of_experts", MixtureOfExperts)

@@ -35,4 +35,20 @@ class RMSNorm(Norm):
         return self.weight, self.eps
 
 
+class CenteredRMSNorm(RMSNorm):
+    """RMSNorm whose checkpoint stores the weight's distance from one: y = (1 + w) * x / sqrt(mean(x^2) + eps).
+    The sum 1 + w is made once, in 32-bit, when the tensor is loaded; from there on this is the plain formula
+    with a 32-bit weight, and every kernel that applies that formula may stand in."""
+
+    def param_specs(self):
+        return {self.tensor: ParamSpec((self.size,), "linear")}
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        self.weight = placement.place(get(self.tensor), torch.float32).add_(1.0)
+
+    def fused_rms(self):
+        return self.weight, self.eps
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "rmsnorm_centered", CenteredRMSNorm)
