@@ -93,6 +93,28 @@ def rilonex_at(width: int, ff: int, heads: int, layers: int, vocab: int, streams
             "layers": [kinds[order[i % len(order)]] for i in range(layers)]}
 
 
+def bidirax_at(width: int, ff: int, heads: int, layers: int, vocab: int, only: str = "") -> dict:
+    """Bidirax layers of a Llama layer's width, heads and active feed-forward size: rotated latent attention with a dense
+    feed-forward, then windowed latent attention with 16 experts (2 a token, a quarter of the feed-forward size each, beside a
+    shared one of half of it), the second of them reading the first one's latent."""
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 2, "scale": 1.0}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2}}
+    rot = {"base": 10000.0, "dims": 32, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    full = {"heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 256, "q_rank": width // 2, "scale": 96 ** -0.5, "rot": rot}
+    win = {"heads": heads, "dim": 64, "vdim": 64, "kv_rank": 256, "q_rank": width // 2, "scale": 0.125, "mask": {"size": 1024}}
+    out = []
+    for i in range(layers):
+        kind = only or ("rotated", "windowed", "windowed_shared")[i % 3]
+        if kind == "rotated":
+            out.append({"type": "latent_attention", "mixer": full, "mlp": dense})
+        elif kind == "windowed" or not out or out[-1]["type"] != "latent_attention_2" or "kv_from" in out[-1]["mixer"]:
+            out.append({"type": "latent_attention_2", "mixer": win, "mlp": moe})
+        else:
+            out.append({"type": "latent_attention_2", "mixer": dict(win, kv_from=i - 1), "mlp": moe})
+    return {"architecture": "Bidirax", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+            "layers": out}
+
+
 def design(args) -> int:
     """Prefill (one prompt of --prefill-tokens) and decode (--batch requests at --context) of the Rilonex design and of
     Llama with layers of the same width, feed-forward size and number of heads: tokens/s of both and their ratio, per
@@ -105,8 +127,11 @@ def design(args) -> int:
     for size in [x for x in args.design_sizes.split(",") if x]:
         width, ff, heads = DESIGN_SIZES[size]
         row = {"size": size, "width": width, "ff": ff, "heads": heads, "layers": layers}
-        for name, cfg in (("llama", llama_at(width, ff, heads, layers, vocab)),
-                          ("rilonex", rilonex_at(width, ff, heads, layers, vocab, only=args.design_only))):
+        other = (bidirax_at(width, ff, heads, layers, vocab, only=args.design_only) if args.design == "bidirax"
+                 else rilonex_at(width, ff, heads, layers, vocab, only=args.design_only))
+        for name, cfg in (("llama", llama_at(width, ff, heads, layers, vocab)), (args.design, other)):
+            if args.design_skip_llama and name == "llama":
+                continue
             engine = Engine.from_random(cfg, args.seed, args.dtype, std=0.02)
             gen = torch.Generator().manual_seed(args.seed + 1)
             prompt = torch.randint(0, vocab, (T,), generator=gen).tolist()
@@ -142,13 +167,14 @@ def design(args) -> int:
             log(f"{size} {name}: prefill {T} tokens {pre_ms:.2f} ms, decode b{batch} ctx {args.context} {dec_ms:.3f} ms/step")
             del cache, engine
             torch.cuda.empty_cache()
-        row["prefill_ratio"] = round(row["rilonex"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3)
-        row["decode_ratio"] = round(row["rilonex"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3)
+        if "llama" in row:
+            row["prefill_ratio"] = round(row[args.design]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3)
+            row["decode_ratio"] = round(row[args.design]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3)
         rows.append(row)
     print(json.dumps({"metric": "design_tokens_per_second_beside_llama", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype,
-                      "value": rows[0]["rilonex"]["decode_tok_s"] if rows else None,
+                      "value": rows[0][args.design]["decode_tok_s"] if rows else None, "design": args.design,
                       "config": {"prefill_tokens": T, "batch": args.batch, "context": args.context, "page_size": page,
-                                 "vocab": vocab, "only": args.design_only or "rglru, channel_delta, parallel in turn"},
+                                 "vocab": vocab, "only": args.design_only or "every kind of layer in turn"},
                       "sizes": rows}), flush=True)
     return 0
 
@@ -345,8 +371,10 @@ def main() -> int:
                          "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
                          "portion beside one decoded token of --batch other requests")
     ap.add_argument("--design-sizes", default="1k,2k", help="design: sizes to run, of " + ",".join(sorted(DESIGN_SIZES)))
-    ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel"],
-                    help="design: a Rilonex of this kind of layer only")
+    ap.add_argument("--design", default="rilonex", choices=["rilonex", "bidirax"], help="design: which design runs beside Llama")
+    ap.add_argument("--design-only", default="", choices=["", "rglru", "channel_delta", "parallel", "rotated", "windowed"],
+                    help="design: a model of this kind of layer only (the first three Rilonex, the others Bidirax)")
+    ap.add_argument("--design-skip-llama", action="store_true", help="design: time the design alone")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--decode-len", type=int, default=700, help="mixed: tokens of the shortest decoding request "
                                                                 "(the longest has 800 more)")

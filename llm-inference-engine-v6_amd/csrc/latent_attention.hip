@@ -245,7 +245,7 @@ extern "C" int llme_latent_prepare(const float* p, int ldp, int Rq, int R, int r
 extern "C" int llme_latent_q_rotate(const void* q, int dtype, const float* freq, float mag, const int* positions,
                                     void* qp, int T, int n, int d, int r, int rd, int R, hipStream_t stream) {
     if (T <= 0 || r == 0) return 0;
-    if (r % 2 || rd < 0 || rd > r || rd % 2 || n <= 0 || d < 0 || R <= 0 || (rd > 0 && freq == nullptr)) return kErrBadArgument;
+    if (r % 2 || rd < 0 || rd > r || rd % 2 || n <= 0 || d < 0 || R < 0 || (rd > 0 && freq == nullptr)) return kErrBadArgument;
     const size_t total = static_cast<size_t>(T) * n * (r / 2);
     const dim3 grid(static_cast<unsigned>((total + 255) / 256));
     if (dtype == kF32)

@@ -33,6 +33,7 @@ HIPCC_FLAGS = [
 SOURCE_FLAGS = {
     "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "latent_attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

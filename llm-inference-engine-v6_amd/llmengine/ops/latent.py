@@ -140,6 +140,85 @@ def latent_attention(qp: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, s
           "latent_attention")
 
 
+# --- latent attention on the matrix cores ------------------------------------------------
+declare("llme_latent_attention_mfma", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i,
+                                       _l, _l, _l, _l, _vp])
+declare("llme_latent_q_split", [_vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+declare("llme_heads_to_rows", [_vp, _vp, _i, _i, _i, _vp])
+LATENT_MFMA_MAX_ROW, LATENT_MFMA_MAX_RANK = 576, 512
+
+
+def latent_mfma_fits(cache: torch.Tensor, kv_rank: int, rot: int, choices=None) -> bool:
+    """Whether the matrix-core kernel takes these rows: bfloat16, a latent that is a multiple of 16, rows a multiple of 32,
+    pages a multiple of 16."""
+    from .choices import DEFAULT
+    D = kv_rank + rot
+    return ((choices or DEFAULT).fast_attention and cache.dtype == torch.bfloat16 and kv_rank % 16 == 0 and D % 32 == 0 and rot % 8 == 0
+            and cache.shape[1] % 16 == 0 and D <= LATENT_MFMA_MAX_ROW and kv_rank <= LATENT_MFMA_MAX_RANK)
+
+
+def latent_splits(step, heads: int, window: int) -> tuple[int, int]:
+    """(the most tokens a request brings, runs to cut the keys into) for the matrix-core kernel: enough workgroups for two a
+    compute unit, runs of 64 keys at least. A step of single tokens plans for requests of up to step.plan_len keys where that
+    is set (the step may be recorded and replayed for longer requests)."""
+    from . import mfma
+    decode = step.num_tokens == step.num_seqs
+    max_new = 1 if decode else max(step.new_lens)
+    if decode and step.plan_len is not None:
+        keys = step.plan_len
+    else:
+        keys = max(c + n for c, n in zip(step.ctx_lens, step.new_lens))
+    if window:
+        keys = min(keys, window + max_new)
+    groups = (max_new * heads + 63) // 64 * step.num_seqs
+    return max_new, max(1, min(32, (2 * mfma.compute_units()) // groups, (keys + 63) // 64))
+
+
+def latent_attention_mfma(qa: torch.Tensor, qr: torch.Tensor | None, cache: torch.Tensor, out: torch.Tensor, step,
+                          block_table: torch.Tensor, heads: int, kv_rank: int, scale: float, window: int, head_major: bool) -> None:
+    """The matrix-core kernel. qa [T, heads, kv_rank] and qr [T, heads, rot] (head_major: [heads, T, ..]); out as qa."""
+    T = step.num_tokens
+    D = cache.shape[2]
+    rot = D - kv_rank
+    require(cache, "cache", torch.bfloat16, (None, None, D))
+    require(qa, "qa", torch.bfloat16)
+    require(out, "out", torch.bfloat16)
+    if qa.numel() != T * heads * kv_rank or out.numel() != qa.numel() or (rot and (qr is None or qr.numel() != T * heads * rot)):
+        raise KernelError("latent attention: the queries do not fit the step")
+    if rot:
+        require(qr, "qr", torch.bfloat16)
+    max_new, nsplit = latent_splits(step, heads, window)
+    ws_o = ws_ml = None
+    if nsplit > 1:
+        ws_o = step.buffer("latent.split_sums", (nsplit, heads * T, kv_rank), torch.float32)
+        ws_ml = step.buffer("latent.split_stats", (nsplit, heads * T, 2), torch.float32)
+    ts, hs = (1, T) if head_major else (heads, 1)
+    check(entry("llme_latent_attention_mfma")(
+        ptr(qa), ptr(qr) if rot else None, ptr(cache), ptr(out), ptr(ws_o), ptr(ws_ml), ptr(step.positions), ptr(step.q_start),
+        ptr(block_table), block_table.shape[1], T, step.num_seqs, max_new, heads, kv_rank, rot, cache.shape[1], float(scale),
+        int(window), nsplit, ts, hs, ts, hs, stream()), "latent_attention_mfma")
+
+
+def latent_q_split(q: torch.Tensor, freq: torch.Tensor | None, mag: float, positions: torch.Tensor, qn: torch.Tensor,
+                   qr: torch.Tensor | None, heads: int, dim: int, rot: int, rot_dims: int) -> None:
+    """q [T, heads (dim + rot)] -> qn [heads, T, dim], the unrotated entries, and qr [heads, T, rot], the rotated ones."""
+    T = q.shape[0]
+    require(q, "q", torch.bfloat16, (T, heads * (dim + rot)))
+    require(qn, "qn", torch.bfloat16, (heads, T, dim))
+    if rot:
+        require(qr, "qr", torch.bfloat16, (heads, T, rot))
+    check(entry("llme_latent_q_split")(ptr(q), ptr(freq) if rot_dims else None, float(mag), ptr(positions), ptr(qn),
+                                       ptr(qr) if rot else None, T, heads, dim, rot, rot_dims, stream()), "latent_q_split")
+
+
+def heads_to_rows(o: torch.Tensor, out: torch.Tensor) -> None:
+    """o [heads, T, c] -> out [T, heads * c]."""
+    require(o, "o", torch.bfloat16, (None, None, None))
+    n, T, c = o.shape
+    require(out, "out", torch.bfloat16, (T, n * c))
+    check(entry("llme_heads_to_rows")(ptr(o), ptr(out), T, n, c, stream()), "heads_to_rows")
+
+
 # --- mixture of experts ----------------------------------------------------------------
 def moe_capacity(pairs: int, experts: int) -> int:
     """Places for `pairs` (token, expert) pairs when every expert's run is padded to whole tiles."""

@@ -131,12 +131,20 @@ class LatentAttention(Mixer):
                            step, table, cq, rows, self.eps)
         q = step.buffer("latent.q", (T, n * (d + r)), act)
         ops.gemm(cq, self.w_uq, q, choices=step.choices)
-        qp = step.buffer("latent.qp", (T, n * D), act)
-        ops.head_gemm(q, d + r, self.w_uk_t, qp, D, n, choices=step.choices)
-        if r:
-            ops.latent_q_rotate(q, self.freq, self.mag, step.positions, qp, n, d, r, self.rot_dims, R)
         ol = step.buffer("latent.sum", (T, n * R), act)
-        ops.latent_attention(qp, rows, ol, step, table, n, R, self.scale, self.window)
+        if ops.latent.latent_mfma_fits(rows, R, r, step.choices) and act == torch.bfloat16:
+            qa = step.buffer("latent.qa", (T, n * R), act)
+            ops.head_gemm(q, d + r, self.w_uk_t, qa, R, n, choices=step.choices)
+            qr = step.buffer("latent.qr", (T, n * r), act) if r else None
+            if r:
+                ops.latent_q_rotate(q, self.freq, self.mag, step.positions, qr, n, d, r, self.rot_dims, 0)
+            ops.latent.latent_attention_mfma(qa, qr, rows, ol, step, table, n, R, self.scale, self.window, head_major=False)
+        else:
+            qp = step.buffer("latent.qp", (T, n * D), act)
+            ops.head_gemm(q, d + r, self.w_uk_t, qp, D, n, choices=step.choices)
+            if r:
+                ops.latent_q_rotate(q, self.freq, self.mag, step.positions, qp, n, d, r, self.rot_dims, R)
+            ops.latent_attention(qp, rows, ol, step, table, n, R, self.scale, self.window)
         o = step.buffer("latent.o", (T, n * dv), act)
         ops.head_gemm(ol, R, self.w_uv, o, dv, n, choices=step.choices)
         ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
