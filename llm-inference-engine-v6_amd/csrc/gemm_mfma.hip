@@ -52,13 +52,31 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 constexpr int kBufferFlags = 0x00020000;
 
 enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4, kRopeCache = 5,
-                     kGatedReluBF16 = 6 };
-// The gated outputs: act(gate) * up with act = SiLU (kGatedBF16) or the rectifier (kGatedReluBF16).
-constexpr bool is_gated(int mode) { return mode == kGatedBF16 || mode == kGatedReluBF16; }
+                     kGatedReluBF16 = 6, kGatedGeluBF16 = 7 };
+// The gated outputs: act(gate) * up with act = SiLU (kGatedBF16), the rectifier (kGatedReluBF16) or the tanh form of
+// GELU (kGatedGeluBF16).
+constexpr bool is_gated(int mode) { return mode == kGatedBF16 || mode == kGatedReluBF16 || mode == kGatedGeluBF16; }
 template <int MODE> __device__ __forceinline__ float gate_act(float g) {
     if (MODE == kGatedReluBF16) return fmaxf(g, 0.f);
+    if (MODE == kGatedGeluBF16) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     return g / (1.0f + expf(-g));
 }
+
+// Products in groups (the tile kernel's GROUPED instances): every row tile belongs to one group and is multiplied by that
+// group's matrix, w + group * w_stride.
+//  * tile_group given (experts): tile t holds rows t BM .. of `out`; its group is tile_group[t]; tiles from n_tiles[0] on do
+//    not exist; row m of `a` is row_index[m] / gather_div where row_index is given (a negative entry: a row of zeros).
+//  * otherwise (heads): every group has rows_per_group rows of `a` and `out`, one group after the other, in tiles_per_group
+//    tiles.
+struct Groups {
+    const int* tile_group = nullptr;
+    const int* n_tiles = nullptr;
+    const int* row_index = nullptr;
+    int gather_div = 1;
+    int rows_per_group = 0, tiles_per_group = 1;
+    long w_stride = 0;          // elements
+    unsigned a_bytes = 0;       // of the whole of `a`, where rows are gathered
+};
 
 // Where the q/k/v projection's epilogue (kRopeCache) puts its result: the columns are the heads
 // of q, then k, then v (hd columns each); q and k heads are rotated at the rows' positions (pairs
@@ -343,10 +361,10 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
 // kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
 // columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
 // silu(gate) * up (src/engine.cpp:213-216).
-template <int WMT, int WNT, int MODE, bool KFULL, bool BLOCKED>
+template <int WMT, int WNT, int MODE, bool KFULL, bool BLOCKED, bool GROUPED = false>
 __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
-                                                        int tiles_m, int tiles_n, int ksplit, QkvTarget qt) {
+                                                        int tiles_m, int tiles_n, int ksplit, QkvTarget qt, Groups gr) {
     constexpr int BM = 32 * WMT, BN = 32 * WNT;
     constexpr int A_ELEMS = BM * TSTRIDE, W_ELEMS = BN * TSTRIDE;
     constexpr int CA = BM / 32, CW = BN / 32;        // 16-byte chunks per thread and slab
@@ -371,7 +389,20 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
     const int tm = first_m + (pid % per_group) % gsize;
     const int tn = (pid % per_group) / gsize;
-    const int m0 = tm * BM, n0 = tn * BN;
+    int m0 = tm * BM;
+    const int n0 = tn * BN;
+    if (GROUPED) {
+        if (gr.n_tiles != nullptr && tm >= gr.n_tiles[0]) return;
+        int group;
+        if (gr.tile_group != nullptr) {
+            group = gr.tile_group[tm];
+        } else {
+            group = tm / gr.tiles_per_group;
+            m0 = group * gr.rows_per_group + (tm % gr.tiles_per_group) * BM;
+            M = (group + 1) * gr.rows_per_group;
+        }
+        w += static_cast<size_t>(group) * gr.w_stride;
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -394,13 +425,23 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     // span fewer than 2^32 bytes: the entry point checks K.)
     const int crow = tid >> 3, ckq = (tid & 7) * 8;   // chunk i of a thread: row crow + 32 i, same k offset
     const int a_rows = M - m0 < BM ? M - m0 : BM, w_rows = N - n0 < BN ? N - n0 : BN;
+    const bool gathered = GROUPED && gr.row_index != nullptr;
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16*>(a + static_cast<size_t>(m0) * K), 0, a_rows * K * 2, kBufferFlags);
+        const_cast<bf16*>(gathered ? a : a + static_cast<size_t>(m0) * K), 0, gathered ? gr.a_bytes : a_rows * K * 2, kBufferFlags);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16*>(w + static_cast<size_t>(n0) * K), 0, w_rows * K * 2, kBufferFlags);
     unsigned aoff[CA], woff[CW];                      // bytes
 #pragma unroll
     for (int i = 0; i < CA; ++i) aoff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
+    if (gathered) {
+        // (a row that is no row lies behind the descriptor's end and reads as zeros)
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            const int m = m0 + crow + 32 * i;
+            const int src = m < M ? gr.row_index[m] : -1;
+            aoff[i] = src < 0 ? gr.a_bytes : (static_cast<unsigned>(src / gr.gather_div) * K + ckq) * 2;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < CW; ++i) woff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
     // Blocked W: a slab of the tile is (BN / 16) row groups x 2 blocks of 1 KB; chunk c = 256 i + t of
@@ -602,7 +643,7 @@ __device__ __forceinline__ void load_b128_to_lds(u32x4 rsrc, unsigned lds_base, 
 template <int WR, int WC, int WMT, int WNT, int MODE>
 __global__ __launch_bounds__(64 * WR * WC, 1) void gemm_tile_direct_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, void* __restrict__ out, int M, int N, int K, int tiles_m,
-    int tiles_n, int ksplit, QkvTarget qt) {
+    int tiles_n, int ksplit, QkvTarget qt, Groups) {        // (no grouped instances: the argument keeps the launches alike)
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NW = WR * WC;
     constexpr int AC = BM / 8, WB = BN / 16;                    // loads: chunks of a slab of A, blocks of half a slab of W
     static_assert(AC % NW == 0 && WB % NW == 0, "every wavefront has the same loads");
@@ -751,8 +792,39 @@ static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(THREADS), LDS, stream, A, W, out, M, N, K, tiles_m,
-                       tiles_n, ksplit, qt);
+                       tiles_n, ksplit, qt, Groups{});
     return launch_status();
+}
+
+// The tile kernel's grouped instances (see Groups): row-major matrices, k whole or not, one of three epilogues.
+template <int WMT, int WNT, int MODE>
+static int launch_grouped_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int tiles_m, const Groups& gr,
+                               hipStream_t stream) {
+    constexpr int LDS = tile_lds_bytes<WMT, WNT>(), BN = 32 * WNT;
+    const int tiles_n = (N + BN - 1) / BN;
+    auto go = [&](auto kernel) -> int {
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+            if (e != hipSuccess) return static_cast<int>(e);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m, tiles_n, 1,
+                           QkvTarget{}, gr);
+        return launch_status();
+    };
+    if (K % TK != 0) return go(&gemm_tile_kernel<WMT, WNT, MODE, false, false, true>);
+    return go(&gemm_tile_kernel<WMT, WNT, MODE, true, false, true>);
+}
+template <int WMT, int WNT>
+static int launch_grouped(const bf16* A, const bf16* W, void* out, int M, int N, int K, int mode, int tiles_m, const Groups& gr,
+                          hipStream_t stream) {
+    switch (mode) {
+        case kStoreF32: return launch_grouped_mode<WMT, WNT, kStoreF32>(A, W, out, M, N, K, tiles_m, gr, stream);
+        case kGatedBF16: return launch_grouped_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, tiles_m, gr, stream);
+        case kStoreBF16: return launch_grouped_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, tiles_m, gr, stream);
+        default: return kErrBadArgument;
+    }
 }
 
 template <int WMT, int WNT, int MODE, bool BLOCKED>
@@ -782,6 +854,7 @@ static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, in
         case kAtomicF32: return launch_tile_mode<WMT, WNT, kAtomicF32>(A, W, out, M, N, K, ksplit, blocked, stream);
         case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, blocked, stream);
         case kGatedReluBF16: return launch_tile_mode<WMT, WNT, kGatedReluBF16>(A, W, out, M, N, K, 1, blocked, stream);
+        case kGatedGeluBF16: return launch_tile_mode<WMT, WNT, kGatedGeluBF16>(A, W, out, M, N, K, 1, blocked, stream);
         default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, blocked, stream);
     }
 }
@@ -800,6 +873,7 @@ static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, in
         case kAtomicF32: return LLME_DIRECT(kAtomicF32);
         case kGatedBF16: return LLME_DIRECT(kGatedBF16);
         case kGatedReluBF16: return LLME_DIRECT(kGatedReluBF16);
+        case kGatedGeluBF16: return LLME_DIRECT(kGatedGeluBF16);
         default: return LLME_DIRECT(kStoreBF16);
     }
 #undef LLME_DIRECT
@@ -991,7 +1065,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // tile shape: 0 lets the entry point choose: the largest tile that still gives about one
     // workgroup per compute unit; a small output with a long k is cut over k instead (the
     // parts are added with atomics, so this needs an accumulating float32 output).
-    if (gated) mode = gated == 2 ? kGatedReluBF16 : kGatedBF16;
+    if (gated) mode = gated == 2 ? kGatedReluBF16 : gated == 3 ? kGatedGeluBF16 : kGatedBF16;
     const bool auto_shape = tile_shape <= 0;
     float tiles_cost = -1.f;                           // of the chosen tile, in the units of the estimate below
     if (tile_shape <= 0) {
@@ -1091,6 +1165,45 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     return kErrBadArgument;
+}
+
+// Products in groups on the tile kernel (see Groups). a [a_rows, K], w [groups, N, K] row-major, both bfloat16.
+// Experts (tile_group given): `out` has max_tiles * tile rows, row tile t belongs to expert tile_group[t] and exists if
+// t < n_tiles[0]; row m of a tile is row row_index[m] / gather_div of `a` (row_index null: row m itself; negative: zeros).
+// Heads (tile_group null): group g owns rows g * rows_per_group .. of `a` and of `out`.
+// gated: w holds gate and up rows interleaved in groups of 16, out [.., N / 2] = silu(gate) * up. tile: 64 or 128 rows.
+extern "C" int llme_gemm_bf16_grouped(const void* a, const void* w, void* out, int out_dtype, int gated, int N, int K, int tile,
+                                      int max_tiles, const int* tile_group, const int* n_tiles, const int* row_index,
+                                      int gather_div, long a_rows, int groups, int rows_per_group, hipStream_t stream) {
+    if (N <= 0 || groups <= 0) return 0;
+    if (K <= 0 || K % 8 != 0 || K >= (1 << 23) || (tile != 64 && tile != 128)) return kErrUnsupported;
+    if (out_dtype != kF32 && out_dtype != kBF16) return kErrBadArgument;
+    if (gated && (out_dtype != kBF16 || N % 32 != 0)) return kErrBadArgument;
+    if (a_rows * K * 2 >= (1l << 32) - 65536) return kErrUnsupported;
+    Groups gr;
+    gr.w_stride = static_cast<long>(N) * K;
+    int tiles_m, M;
+    if (tile_group != nullptr) {
+        if (max_tiles <= 0) return 0;
+        gr.tile_group = tile_group;
+        gr.n_tiles = n_tiles;
+        gr.row_index = row_index;
+        gr.gather_div = gather_div > 0 ? gather_div : 1;
+        gr.a_bytes = static_cast<unsigned>(a_rows * K * 2);
+        tiles_m = max_tiles;
+        M = max_tiles * tile;
+    } else {
+        if (rows_per_group <= 0) return 0;
+        gr.rows_per_group = rows_per_group;
+        gr.tiles_per_group = (rows_per_group + tile - 1) / tile;
+        tiles_m = groups * gr.tiles_per_group;
+        M = groups * rows_per_group;
+    }
+    const int mode = gated ? kGatedBF16 : out_dtype == kBF16 ? kStoreBF16 : kStoreF32;
+    const bf16* A = static_cast<const bf16*>(a);
+    const bf16* W = static_cast<const bf16*>(w);
+    if (tile == 128) return launch_grouped<4, 4>(A, W, out, M, N, K, mode, tiles_m, gr, stream);
+    return launch_grouped<2, 2>(A, W, out, M, N, K, mode, tiles_m, gr, stream);
 }
 
 // The q/k/v projection of many rows (prompts) with rotation and cache write in its epilogue:

@@ -8,7 +8,8 @@
 //                of tiles. One workgroup; which place of its expert's run a pair takes depends on the
 //                order of atomics, which no result depends on (every place is computed on its own).
 //   moe_gemm     per tile of places: rows gathered (token = pair / top, or the place itself) times the
-//                tile's expert's matrix [N, K]; plain or gated (act(gate) * up of two matrices)
+//                tile's expert's matrix [N, K]; plain or gated (act(gate) * up, gate and up rows in one matrix);
+//                the plain-precision kernel; bfloat16 steps take the grouped instances of the matrix-core tile kernel
 //   moe_combine  out[t] (+)= sum_k weight[t, k] * y[place of (t, k)], k in order
 //
 // Everything that depends on the routing is read from device memory: a step's launches are the same
@@ -125,29 +126,31 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     (void)used;
 }
 
-// Tiles of 16 places x 64 columns, k in slabs of 32 through LDS, 32-bit sums. GATED: out = act(a . wg) * (a . wu).
-// gather_div > 0: row of `a` = pair / gather_div (the token); 0: the place itself. Rows of padding give zeros.
+// Pieces of 16 places x 64 columns (a tile of `tile` places is tile / 16 pieces), k in slabs of 32 through LDS, 32-bit
+// sums. GATED: out = act(a . gate) * (a . up), the expert's matrix holding gate and up rows in alternating groups of
+// `group` rows (2 N rows in all). gather_div > 0: row of `a` = pair / gather_div (the token); 0: the place itself.
+// Rows of padding give zeros.
 template <typename TA, typename TW, typename TO, bool GATED>
-__global__ __launch_bounds__(256) void moe_gemm_kernel(const TA* __restrict__ a, const TW* __restrict__ w,
-                                                       const TW* __restrict__ w2, TO* __restrict__ out,
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO* __restrict__ out,
                                                        const int* __restrict__ place_pair, const int* __restrict__ tile_expert,
-                                                       const int* __restrict__ n_tiles, int gather_div, int N, int K, int act) {
+                                                       const int* __restrict__ n_tiles, int tile, int gather_div, int N, int K,
+                                                       int group, int act) {
     __shared__ float As[16][33];
     __shared__ float Ws[64][33];
     __shared__ float Us[GATED ? 64 : 1][33];
     __shared__ int rows[16];
-    const int tile = blockIdx.y;
-    if (tile >= n_tiles[0]) return;
+    const int piece = blockIdx.y;
+    const int big = piece * 16 / tile;
+    if (big >= n_tiles[0]) return;
     const int n0 = blockIdx.x * 64;
-    const int e = tile_expert[tile];
+    const int e = tile_expert[big];
     if (threadIdx.x < 16) {
-        const int pair = place_pair[tile * 16 + threadIdx.x];
-        rows[threadIdx.x] = pair < 0 ? -1 : (gather_div > 0 ? pair / gather_div : tile * 16 + threadIdx.x);
+        const int pair = place_pair[piece * 16 + threadIdx.x];
+        rows[threadIdx.x] = pair < 0 ? -1 : (gather_div > 0 ? pair / gather_div : piece * 16 + threadIdx.x);
     }
     __syncthreads();
     const int tr = threadIdx.x / 16, tc = threadIdx.x % 16;
-    const TW* we = w + static_cast<size_t>(e) * N * K;
-    const TW* ue = GATED ? w2 + static_cast<size_t>(e) * N * K : nullptr;
+    const TW* we = w + static_cast<size_t>(e) * (GATED ? 2 : 1) * N * K;
     float acc[4] = {0.f, 0.f, 0.f, 0.f}, acu[4] = {0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < K; k0 += 32) {
         for (int i = threadIdx.x; i < 16 * 32; i += 256) {
@@ -159,8 +162,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const TA* __restrict__ a,
             const int nn = i / 32, kk = i % 32;
             const int n = n0 + nn, k = k0 + kk;
             const bool in = n < N && k < K;
-            Ws[nn][kk] = in ? to_float(we[static_cast<size_t>(n) * K + k]) : 0.f;
-            if (GATED) Us[nn][kk] = in ? to_float(ue[static_cast<size_t>(n) * K + k]) : 0.f;
+            const size_t row = GATED ? static_cast<size_t>(n / group) * 2 * group + n % group : n;      // the gate's row; up: group further
+            Ws[nn][kk] = in ? to_float(we[row * K + k]) : 0.f;
+            if (GATED) Us[nn][kk] = in ? to_float(we[(row + group) * K + k]) : 0.f;
         }
         __syncthreads();
 #pragma unroll 8
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const TA* __restrict__ a,
         }
         __syncthreads();
     }
-    TO* orow = out + (static_cast<size_t>(tile) * 16 + tr) * N;
+    TO* orow = out + (static_cast<size_t>(piece) * 16 + tr) * N;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int n = n0 + tc + 16 * j;
@@ -220,22 +224,24 @@ extern "C" int llme_moe_plan(const int* ids, int pairs, int E, int tile, int cap
     return launch_status();
 }
 
-extern "C" int llme_moe_gemm(const void* a, int a_dtype, const void* w, const void* w2, int w_dtype, void* out,
-                             int out_dtype, const int* place_pair, const int* tile_expert, const int* n_tiles,
-                             int max_tiles, int gather_div, int N, int K, int act, hipStream_t stream) {
+// gated: w [experts, 2 N, K] with gate and up rows in alternating groups of `group`; else w [experts, N, K].
+extern "C" int llme_moe_gemm(const void* a, int a_dtype, const void* w, int gated, int w_dtype, void* out,
+                             int out_dtype, const int* place_pair, const int* tile_expert, const int* n_tiles, int tile,
+                             int max_tiles, int gather_div, int N, int K, int group, int act, hipStream_t stream) {
     if (max_tiles <= 0 || N <= 0) return 0;
-    if (K <= 0 || max_tiles > 65535) return kErrUnsupported;
-    const dim3 grid((N + 63) / 64, max_tiles);
+    if (tile <= 0 || tile % 16 || (gated && (group <= 0 || N % group))) return kErrBadArgument;
+    if (K <= 0 || static_cast<long>(max_tiles) * (tile / 16) > 65535) return kErrUnsupported;
+    const dim3 grid((N + 63) / 64, max_tiles * (tile / 16));
 #define LLME_MG(TA, TW, TO)                                                                                      \
     do {                                                                                                         \
-        if (w2 != nullptr)                                                                                       \
+        if (gated)                                                                                               \
             hipLaunchKernelGGL((moe_gemm_kernel<TA, TW, TO, true>), grid, dim3(256), 0, stream,                  \
-                               static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<const TW*>(w2), \
-                               static_cast<TO*>(out), place_pair, tile_expert, n_tiles, gather_div, N, K, act);  \
+                               static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<TO*>(out),      \
+                               place_pair, tile_expert, n_tiles, tile, gather_div, N, K, group, act);            \
         else                                                                                                     \
             hipLaunchKernelGGL((moe_gemm_kernel<TA, TW, TO, false>), grid, dim3(256), 0, stream,                 \
-                               static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<const TW*>(w2), \
-                               static_cast<TO*>(out), place_pair, tile_expert, n_tiles, gather_div, N, K, act);  \
+                               static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<TO*>(out),      \
+                               place_pair, tile_expert, n_tiles, tile, gather_div, N, K, group, act);            \
     } while (0)
     if (a_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) LLME_MG(float, float, float);
     else if (a_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) LLME_MG(bf16, bf16, bf16);

@@ -23,7 +23,7 @@ declare("llme_head_gemm", [_vp, _i, _l, _l, _vp, _i, _vp, _i, _l, _l, _i, _i, _i
 declare("llme_latent_attention", [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp])
 declare("llme_moe_route", [_vp, _i, _i, _i, _f, _i, _vp, _vp, _vp])
 declare("llme_moe_plan", [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp])
-declare("llme_moe_gemm", [_vp, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+declare("llme_moe_gemm", [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 declare("llme_moe_combine", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp])
 
 
@@ -219,10 +219,48 @@ def heads_to_rows(o: torch.Tensor, out: torch.Tensor) -> None:
     check(entry("llme_heads_to_rows")(ptr(o), ptr(out), T, n, c, stream()), "heads_to_rows")
 
 
+# --- products in groups on the matrix cores -------------------------------------------------
+declare("llme_gemm_bf16_grouped", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _l, _i, _i, _vp])
+
+
+def _grouped_fits(a: torch.Tensor, w: torch.Tensor, choices) -> bool:
+    from .choices import DEFAULT
+    return ((choices or DEFAULT).fast_gemm and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[-1] % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and a.numel() * 2 < (1 << 32) - 65536)
+
+
+def heads_gemm_fits(a: torch.Tensor, w: torch.Tensor, choices=None) -> bool:
+    return _grouped_fits(a, w, choices)
+
+
+def heads_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[h] = a[h] w[h]^T for a [heads, T, K], w [heads, N, K], out [heads, T, N], all bfloat16: the matrix-core tile
+    kernel with a matrix per group of row tiles."""
+    require(a, "a", torch.bfloat16, (None, None, None))
+    n, T, K = a.shape
+    require(w, "w", torch.bfloat16, (n, None, K))
+    N = w.shape[1]
+    require(out, "out", torch.bfloat16, (n, T, N))
+    tile = 128 if T >= 512 else 64
+    check(entry("llme_gemm_bf16_grouped")(ptr(a), ptr(w), ptr(out), code(out.dtype), 0, N, K, tile, 0, None, None, None, 1,
+                                          n * T, n, T, stream()), "heads_gemm")
+
+
 # --- mixture of experts ----------------------------------------------------------------
-def moe_capacity(pairs: int, experts: int) -> int:
+MOE_FAST_TILES = (64, 128)
+
+
+def moe_tile(x: torch.Tensor, w: torch.Tensor, pairs: int, experts: int, group: int, choices=None) -> int:
+    """Rows of a tile for a step's grouped products: 16 for the plain-precision kernel; 64 or 128 on the matrix cores
+    (bfloat16, gate and up rows interleaved in groups of 16)."""
+    if not _grouped_fits(x, w, choices) or group != 16:
+        return MOE_TILE
+    return 128 if pairs >= 512 * experts else 64
+
+
+def moe_capacity(pairs: int, experts: int, tile: int = MOE_TILE) -> int:
     """Places for `pairs` (token, expert) pairs when every expert's run is padded to whole tiles."""
-    return (pairs + experts * (MOE_TILE - 1) + MOE_TILE - 1) // MOE_TILE * MOE_TILE
+    return (pairs + experts * (tile - 1) + tile - 1) // tile * tile
 
 
 def moe_route(logits: torch.Tensor, top: int, scale: float, renormalize: bool, ids: torch.Tensor, wts: torch.Tensor) -> None:
@@ -234,43 +272,43 @@ def moe_route(logits: torch.Tensor, top: int, scale: float, renormalize: bool, i
           "moe_route")
 
 
-def moe_plan(ids: torch.Tensor, experts: int, place_pair: torch.Tensor, pair_place: torch.Tensor,
+def moe_plan(ids: torch.Tensor, experts: int, tile: int, place_pair: torch.Tensor, pair_place: torch.Tensor,
              tile_expert: torch.Tensor, n_tiles: torch.Tensor) -> None:
     require(ids, "ids", torch.int32, (None, None))
     pairs = ids.numel()
-    cap = moe_capacity(pairs, experts)
+    cap = moe_capacity(pairs, experts, tile)
     require(place_pair, "place_pair", torch.int32, (cap,))
     require(pair_place, "pair_place", torch.int32, (pairs,))
-    require(tile_expert, "tile_expert", torch.int32, (cap // MOE_TILE,))
+    require(tile_expert, "tile_expert", torch.int32, (cap // tile,))
     require(n_tiles, "n_tiles", torch.int32, (1,))
-    check(entry("llme_moe_plan")(ptr(ids), pairs, experts, MOE_TILE, cap, ptr(place_pair), ptr(pair_place), ptr(tile_expert),
+    check(entry("llme_moe_plan")(ptr(ids), pairs, experts, tile, cap, ptr(place_pair), ptr(pair_place), ptr(tile_expert),
                                  ptr(n_tiles), stream()), "moe_plan")
 
 
-_fast_moe_gemm = None           # set by ops/latent_mfma.py
-
-
-def moe_gemm(a: torch.Tensor, w: torch.Tensor, w2: torch.Tensor | None, out: torch.Tensor, place_pair: torch.Tensor,
-             tile_expert: torch.Tensor, n_tiles: torch.Tensor, gather_div: int, activation: str = "silu", choices=None) -> None:
-    """Per place: out[place] = w[expert] a[row] (w2 given: act(w a) * (w2 a)); row = pair // gather_div, or the
-    place itself where gather_div is 0. w, w2 [experts, N, K]."""
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, gated: bool, group: int, out: torch.Tensor, place_pair: torch.Tensor,
+             tile_expert: torch.Tensor, n_tiles: torch.Tensor, tile: int, gather_div: int, activation: str = "silu",
+             choices=None) -> None:
+    """Per place: out[place] = w[expert] a[row]; gated: act(gate a) * (up a), w [experts, 2 N, K] holding gate and up rows in
+    alternating groups of `group`. row = pair // gather_div, or the place itself where gather_div is 0."""
     from .recurrent import GATE_ACTIVATIONS
     require(w, "w", _FLOATS, (None, None, None))
-    E, N, K = w.shape
-    if w2 is not None:
-        require(w2, "w2", w.dtype, (E, N, K))
+    E, rows_w, K = w.shape
+    N = rows_w // 2 if gated else rows_w
     require(a, "a", _FLOATS, (None, K))
     cap = place_pair.shape[0]
     require(out, "out", _FLOATS, (cap, N))
-    require(tile_expert, "tile_expert", torch.int32, (cap // MOE_TILE,))
+    require(tile_expert, "tile_expert", torch.int32, (cap // tile,))
     if gather_div == 0 and a.shape[0] != cap:
         raise KernelError("moe_gemm: rows by place need one row per place")
-    if _fast_moe_gemm is not None and _fast_moe_gemm(a, w, w2, out, place_pair, tile_expert, n_tiles, gather_div,
-                                                     activation, choices):
+    if (tile in MOE_FAST_TILES and _grouped_fits(a, w, choices) and (not gated or (group == 16 and activation == "silu"
+                                                                                  and out.dtype == torch.bfloat16))):
+        check(entry("llme_gemm_bf16_grouped")(ptr(a), ptr(w), ptr(out), code(out.dtype), 1 if gated else 0, rows_w, K, tile,
+                                              cap // tile, ptr(tile_expert), ptr(n_tiles), ptr(place_pair) if gather_div else None,
+                                              max(gather_div, 1), a.shape[0], E, 0, stream()), "moe_gemm")
         return
-    check(entry("llme_moe_gemm")(ptr(a), code(a.dtype), ptr(w), ptr(w2), code(w.dtype), ptr(out), code(out.dtype),
-                                 ptr(place_pair), ptr(tile_expert), ptr(n_tiles), cap // MOE_TILE, int(gather_div), N, K,
-                                 GATE_ACTIVATIONS[activation], stream()), "moe_gemm")
+    check(entry("llme_moe_gemm")(ptr(a), code(a.dtype), ptr(w), 1 if gated else 0, code(w.dtype), ptr(out), code(out.dtype),
+                                 ptr(place_pair), ptr(tile_expert), ptr(n_tiles), tile, cap // tile, int(gather_div), N, K,
+                                 int(group), GATE_ACTIVATIONS[activation], stream()), "moe_gemm")
 
 
 def moe_combine(y: torch.Tensor, pair_place: torch.Tensor, wts: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:

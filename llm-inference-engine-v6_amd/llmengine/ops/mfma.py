@@ -48,7 +48,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     if force_tile and not tile:
         tile = 128
     check(entry("llme_gemm_bf16")(ptr(a), ptr(w), ptr(out), 0 if out.dtype == torch.float32 else 1, M, N, K,
-                                  1 if accumulate else 0, (2 if gated == "relu" else 1) if gated else 0, waves, ksplit, tile,
+                                  1 if accumulate else 0, (2 if gated == "relu" else 3 if gated == "gelu_tanh" else 1) if gated else 0, waves, ksplit, tile,
                                   1 if kernels.is_blocked(w) else 0, int(direct), stream()),
           "gemm_bf16")
 
@@ -61,10 +61,10 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
     activation kernel."""
     T, FF = out.shape
     if ((choices or DEFAULT).fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
-            and activation in ("silu", "relu")
+            and activation in ("silu", "relu", "gelu_tanh")
             and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
         r = tail_rows(T, choices)
-        mode = "relu" if activation == "relu" else True
+        mode = activation if activation in ("relu", "gelu_tanh") else True
         if r:
             gemm_bf16(x[:T - r], w_gate_up, out[:T - r], gated=mode, _supported=True)
             gemm_bf16(x[T - r:], w_gate_up, out[T - r:], gated=mode, _supported=True)

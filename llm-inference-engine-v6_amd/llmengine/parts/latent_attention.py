@@ -132,7 +132,25 @@ class LatentAttention(Mixer):
         q = step.buffer("latent.q", (T, n * (d + r)), act)
         ops.gemm(cq, self.w_uq, q, choices=step.choices)
         ol = step.buffer("latent.sum", (T, n * R), act)
-        if ops.latent.latent_mfma_fits(rows, R, r, step.choices) and act == torch.bfloat16:
+        fast = ops.latent.latent_mfma_fits(rows, R, r, step.choices) and act == torch.bfloat16
+        if (fast and d % 8 == 0 and ops.latent.heads_gemm_fits(q, self.w_uk_t, step.choices)
+                and ops.latent.heads_gemm_fits(ol, self.w_uv, step.choices)):
+            # everything between the up map and the output map with the heads outermost ([heads, T, ..]): the two maps
+            # that differ from head to head are then products of whole row tiles on the matrix cores
+            qn = step.buffer("latent.qn", (n, T, d), act)
+            qr = step.buffer("latent.qr", (n, T, r), act) if r else None
+            ops.latent.latent_q_split(q, self.freq, self.mag, step.positions, qn, qr, n, d, r, self.rot_dims)
+            qa = step.buffer("latent.qa", (n, T, R), act)
+            ops.latent.heads_gemm(qn, self.w_uk_t, qa)
+            ol = ol.view(n, T, R)
+            ops.latent.latent_attention_mfma(qa, qr, rows, ol, step, table, n, R, self.scale, self.window, head_major=True)
+            oh = step.buffer("latent.oh", (n, T, dv), act)
+            ops.latent.heads_gemm(ol, self.w_uv, oh)
+            o = step.buffer("latent.o", (T, n * dv), act)
+            ops.latent.heads_to_rows(oh, o)
+            ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
+            return
+        if fast:
             qa = step.buffer("latent.qa", (T, n * R), act)
             ops.head_gemm(q, d + r, self.w_uk_t, qa, R, n, choices=step.choices)
             qr = step.buffer("latent.qr", (T, n * r), act) if r else None

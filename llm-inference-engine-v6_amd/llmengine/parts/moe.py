@@ -52,11 +52,20 @@ class MixtureOfExperts(FeedForward):
         return out
 
     def load_params(self, get: Getter, placement: Placement) -> None:
-        self.w_router = placement.place(get("router"), torch.float32)
-        names = [self.expert_name.format(e) for e in range(self.experts)]
+        # The router's matrix as the file has it: bfloat16 entries times the bfloat16 input are exact in 32-bit, so the
+        # matrix-core product with its 32-bit sums is the 32-bit product; the 32-bit model widens it like everything else.
+        self.w_router = placement.place(get("router"))
+        E, FF, H = self.experts, self.intermediate_size, self.hidden_size
+        names = [self.expert_name.format(e) for e in range(E)]
         dtype = placement.common_dtype([get(f"{names[0]}.{k}") for k in ("gate", "up", "down")])
-        stack = lambda key: torch.stack([placement.place(get(f"{n}.{key}"), dtype) for n in names]).contiguous()
-        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        # gate and up rows of an expert in alternating groups of 16 in one matrix, as the dense feed-forward keeps them
+        g = self.group = 16 if FF % 16 == 0 else FF
+        self.w_gate_up = torch.empty((E, 2 * FF, H), dtype=dtype, device=placement.device)
+        view = self.w_gate_up.view(E, FF // g, 2, g, H)
+        for e, name in enumerate(names):
+            view[e, :, 0].copy_(get(f"{name}.gate").view(FF // g, g, H))
+            view[e, :, 1].copy_(get(f"{name}.up").view(FF // g, g, H))
+        self.w_down = torch.stack([placement.place(get(f"{n}.down"), dtype) for n in names]).contiguous()
 
     def forward(self, x, step, out, accumulate):
         T, H = x.shape
@@ -66,14 +75,16 @@ class MixtureOfExperts(FeedForward):
         ops.gemm(x, self.w_router, logits, choices=step.choices)
         ids, wts = step.buffer("moe.ids", (T, top), i32), step.buffer("moe.weights", (T, top), f32)
         ops.moe_route(logits, top, self.scale, self.renormalize, ids, wts)
-        cap = ops.moe_capacity(T * top, E)
+        tile = ops.latent.moe_tile(x, self.w_gate_up, T * top, E, self.group, step.choices)
+        cap = ops.moe_capacity(T * top, E, tile)
         place_pair, pair_place = step.buffer("moe.place_pair", (cap,), i32), step.buffer("moe.pair_place", (T * top,), i32)
-        tile_expert, n_tiles = step.buffer("moe.tile_expert", (cap // ops.latent.MOE_TILE,), i32), step.buffer("moe.tiles", (1,), i32)
-        ops.moe_plan(ids, E, place_pair, pair_place, tile_expert, n_tiles)
+        tile_expert, n_tiles = step.buffer("moe.tile_expert", (cap // tile,), i32), step.buffer("moe.tiles", (1,), i32)
+        ops.moe_plan(ids, E, tile, place_pair, pair_place, tile_expert, n_tiles)
         act = step.buffer("moe.act", (cap, FF), step.act_dtype)
-        ops.moe_gemm(x, self.w_gate, self.w_up, act, place_pair, tile_expert, n_tiles, top, self.activation, step.choices)
+        ops.moe_gemm(x, self.w_gate_up, True, self.group, act, place_pair, tile_expert, n_tiles, tile, top, self.activation,
+                     step.choices)
         y = step.buffer("moe.y", (cap, H), f32)
-        ops.moe_gemm(act, self.w_down, None, y, place_pair, tile_expert, n_tiles, 0, self.activation, step.choices)
+        ops.moe_gemm(act, self.w_down, False, 0, y, place_pair, tile_expert, n_tiles, tile, 0, self.activation, step.choices)
         if self.shared is not None:
             self.shared.forward(x, step, out, accumulate)
             accumulate = True
