@@ -238,23 +238,41 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(LatentArgs a
     }
 }
 
-// out[pair] = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, z in order. One workgroup of 64 threads a pair.
-__global__ __launch_bounds__(64) void latent_join_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
-                                                         bf16* __restrict__ out, int T, int n, int R, int nsplit, long o_ts,
-                                                         long o_hs) {
+// out[pair] = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, z in order. One workgroup of 256 threads a pair: the first
+// wavefront turns the runs' statistics into one factor per run (a lane a run, up to 64 runs), then every thread adds its
+// entries of the runs' sums, eight loads asked for at a time.
+__global__ __launch_bounds__(256) void latent_join_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                          bf16* __restrict__ out, int T, int n, int R, int nsplit, long o_ts,
+                                                          long o_hs) {
+    __shared__ float factor[64];
     const int tok = blockIdx.x, h = blockIdx.y;
     const size_t pairs = static_cast<size_t>(n) * T, pair = static_cast<size_t>(h) * T + tok;
-    float M = kLatNoMax;
-    for (int z = 0; z < nsplit; ++z) M = fmaxf(M, ws_ml[(z * pairs + pair) * 2]);
-    float L = 0.f;
-    for (int z = 0; z < nsplit; ++z) L += __builtin_amdgcn_exp2f(ws_ml[(z * pairs + pair) * 2] - M) * ws_ml[(z * pairs + pair) * 2 + 1];
-    const float inv = 1.0f / L;
+    if (threadIdx.x < 64) {
+        const int z = threadIdx.x;
+        const float mz = z < nsplit ? ws_ml[(z * pairs + pair) * 2] : kLatNoMax;
+        const float lz = z < nsplit ? ws_ml[(z * pairs + pair) * 2 + 1] : 0.f;
+        const float M = wave_max(mz);
+        const float f = __builtin_amdgcn_exp2f(mz - M);
+        // (the sum over the runs in the order of the runs: lane 0 adds them up)
+        float L = 0.f;
+        for (int i = 0; i < nsplit; ++i) L += __shfl(f * lz, i, 64);
+        factor[z] = f / L;
+    }
+    __syncthreads();
     bf16* o = out + (static_cast<long>(tok) * o_ts + static_cast<long>(h) * o_hs) * R;
-    for (int c = threadIdx.x; c < R; c += 64) {
+    for (int c = threadIdx.x; c < R; c += 256) {
+        const float* src = ws_o + pair * R + c;
         float sum = 0.f;
-        for (int z = 0; z < nsplit; ++z)
-            sum += __builtin_amdgcn_exp2f(ws_ml[(z * pairs + pair) * 2] - M) * ws_o[(z * pairs + pair) * R + c];
-        o[c] = static_cast<bf16>(sum * inv);
+        int z = 0;
+        for (; z + 8 <= nsplit; z += 8) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = src[static_cast<size_t>(z + e) * pairs * R];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum = fmaf(factor[z + e], v[e], sum);
+        }
+        for (; z < nsplit; ++z) sum = fmaf(factor[z], src[static_cast<size_t>(z) * pairs * R], sum);
+        o[c] = static_cast<bf16>(sum);
     }
 }
 
@@ -327,7 +345,7 @@ extern "C" int llme_latent_attention_mfma(const void* qa, const void* qr, const 
                                           hipStream_t stream) {
     if (T <= 0 || n_seq <= 0) return 0;
     const int D = R + r;
-    if (n <= 0 || R <= 0 || r < 0 || max_new <= 0 || nsplit <= 0 || nsplit > 65535 || n_seq > 65535) return kErrBadArgument;
+    if (n <= 0 || R <= 0 || r < 0 || max_new <= 0 || nsplit <= 0 || nsplit > 64 || n_seq > 65535) return kErrBadArgument;
     if (R % 16 || D % 32 || r % 8 || page % 16 || D > 576 || R > 512) return kErrUnsupported;
     if (static_cast<long>(T) * n * (R > 2 ? R : 2) >= (1l << 31)) return kErrUnsupported;
     if (nsplit > 1 && (ws_o == nullptr || ws_ml == nullptr)) return kErrBadArgument;
@@ -339,7 +357,7 @@ extern "C" int llme_latent_attention_mfma(const void* qa, const void* qr, const 
     else if (D <= 320 && R <= 256) rc = launch_latent<10, 16>(a, max_new, n_seq, stream);
     else rc = launch_latent<18, 32>(a, max_new, n_seq, stream);
     if (rc != 0 || nsplit == 1) return rc;
-    hipLaunchKernelGGL(latent_join_kernel, dim3(T, n), dim3(64), 0, stream, ws_o, ws_ml, static_cast<bf16*>(out), T, n, R, nsplit,
+    hipLaunchKernelGGL(latent_join_kernel, dim3(T, n), dim3(256), 0, stream, ws_o, ws_ml, static_cast<bf16*>(out), T, n, R, nsplit,
                        o_ts, o_hs);
     return launch_status();
 }

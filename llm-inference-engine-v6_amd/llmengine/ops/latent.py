@@ -171,7 +171,7 @@ def latent_splits(step, heads: int, window: int) -> tuple[int, int]:
     if window:
         keys = min(keys, window + max_new)
     groups = (max_new * heads + 63) // 64 * step.num_seqs
-    return max_new, max(1, min(32, (2 * mfma.compute_units()) // groups, (keys + 63) // 64))
+    return max_new, max(1, min(32, (2 * mfma.compute_units()) // groups, (keys + 127) // 128))
 
 
 def latent_attention_mfma(qa: torch.Tensor, qr: torch.Tensor | None, cache: torch.Tensor, out: torch.Tensor, step,
@@ -255,7 +255,7 @@ def moe_tile(x: torch.Tensor, w: torch.Tensor, pairs: int, experts: int, group: 
     (bfloat16, gate and up rows interleaved in groups of 16)."""
     if not _grouped_fits(x, w, choices) or group != 16:
         return MOE_TILE
-    return 128 if pairs >= 512 * experts else 64
+    return 128 if pairs >= 128 * experts else 64
 
 
 def moe_capacity(pairs: int, experts: int, tile: int = MOE_TILE) -> int:
