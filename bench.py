@@ -17,7 +17,8 @@ run at the configured context length. One JSON line goes to stdout.
 measurements at further sizes and context lengths; the default run is the 1B shape).
 
 `--phase design` runs the Rilonex design (recurrent, delta-rule and softmax-free attention layers around
-a residual in several streams) beside Llama with layers of the same sizes: prefill and decode of both.
+a residual in several streams) beside Llama with layers of the same sizes: prefill and decode of both;
+`--design bidirax` the Bidirax design instead (latent attention, rotated and windowed, dense and expert feed-forwards).
 
 `--phase mixed` times one step of continuous batching (a prompt portion beside decoded tokens of
 other requests), `--phase portion` portions of one long prompt. `--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
