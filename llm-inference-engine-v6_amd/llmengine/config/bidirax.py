@@ -134,8 +134,9 @@ class BidiraxConfig:
             other = layers[src].mixer
             if other["kv_from"] is not None:
                 raise ConfigError(f"config.json:layers[{i}]: kv_from={src} names a layer that keeps no latent of its own")
-            if (other["kv_rank"], other["rot_dim"]) != (layer.mixer["kv_rank"], layer.mixer["rot_dim"]):
-                raise ConfigError(f"config.json:layers[{i}]: kv_rank and rot_dim must equal those of layer {src}, whose latent it reads")
+            if other["kv_rank"] != layer.mixer["kv_rank"] or layer.mixer["rot_dim"] not in (0, other["rot_dim"]):
+                raise ConfigError(f"config.json:layers[{i}]: kv_rank must equal that of layer {src}, whose latent it reads "
+                                  "(and rot_dim, unless it is 0)")
         emb = r.mapping("embedding")
         return cls(architecture=architecture, vocab_size=r.integer("vocab", minimum=1), width=r.integer("width", minimum=1),
                    embedding_scale=emb.number("scale", 1.0) if emb is not None else 1.0, norm_eps=norm.number("eps"),

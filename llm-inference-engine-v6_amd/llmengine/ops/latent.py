@@ -50,6 +50,15 @@ def scale_(x: torch.Tensor, s: float) -> None:
     check(entry("llme_scale_f32")(ptr(x), x.numel(), float(s), stream()), "scale")
 
 
+def zero_(t: torch.Tensor) -> None:
+    """Fills a contiguous buffer with zeros (a fill kernel, never a memset: the launch may be recorded)."""
+    from .kernels import clear
+    if t.is_contiguous() and (t.numel() * t.element_size()) % 16 == 0 and t.data_ptr() % 16 == 0:
+        clear(t.view(-1).view(torch.float32))
+    else:
+        t.zero_()
+
+
 # --- latent attention ------------------------------------------------------------------
 def latent_prepare(p: torch.Tensor, q_rank: int, kv_rank: int, rot: int, rot_dims: int, wq: torch.Tensor, wc: torch.Tensor | None,
                    freq: torch.Tensor | None, mag: float, step, block_table: torch.Tensor | None, cq: torch.Tensor,

@@ -10,7 +10,8 @@ the heads' results side by side go through the output matrix.
 Only c and the shared part are cached: a page holds rows of kv_rank + rot_dim entries. The kernels never
 expand a key or a value either: a query takes Wuk_h^T onto itself and is scored against the rows as they
 lie, the weighted sum runs over the rows' latent part, and Wuv_h is applied to that sum. A layer with
-`keeps_latent=False` has no down map for keys and values and reads the rows another layer cached.
+`keeps_latent=False` has no down map for keys and values and reads the rows another layer cached (if those
+rows carry a rotated part and this layer has none, its queries score the latent entries alone).
 
 Rotation: neighbours (2i, 2i + 1) of a part's first `dims` entries turn by position * f_i, with
 f_i = base^(-2i / dims) and, where `scaling` is given, the frequencies blended towards f_i / factor over a ramp
@@ -121,8 +122,12 @@ class LatentAttention(Mixer):
         n, d, r, dv, R, Rq = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self.q_rank
         D, act = R + r, step.act_dtype
         rows = cache.paged["rows"]
-        if rows.shape[2] != D:
+        # A layer without rotated entries may read rows that hold some (the layer that cached them rotates): its queries
+        # have zeros there, so that the rows are scored as they lie.
+        pad = rows.shape[2] - D
+        if pad and (pad < 0 or r or self.keeps_latent):
             raise ValueError(f"the cached rows hold {rows.shape[2]} entries, this layer reads {D}")
+        D += pad
         table = step.block_tables[cache.group]
         p = step.buffer("latent.down", (T, self.down_padded), torch.float32)
         ops.gemm(x, self.w_down, p, choices=step.choices)
@@ -132,14 +137,16 @@ class LatentAttention(Mixer):
         q = step.buffer("latent.q", (T, n * (d + r)), act)
         ops.gemm(cq, self.w_uq, q, choices=step.choices)
         ol = step.buffer("latent.sum", (T, n * R), act)
-        fast = ops.latent.latent_mfma_fits(rows, R, r, step.choices) and act == torch.bfloat16
+        fast = ops.latent.latent_mfma_fits(rows, R, r + pad, step.choices) and act == torch.bfloat16
         if (fast and d % 8 == 0 and ops.latent.heads_gemm_fits(q, self.w_uk_t, step.choices)
                 and ops.latent.heads_gemm_fits(ol, self.w_uv, step.choices)):
             # everything between the up map and the output map with the heads outermost ([heads, T, ..]): the two maps
             # that differ from head to head are then products of whole row tiles on the matrix cores
             qn = step.buffer("latent.qn", (n, T, d), act)
-            qr = step.buffer("latent.qr", (n, T, r), act) if r else None
-            ops.latent.latent_q_split(q, self.freq, self.mag, step.positions, qn, qr, n, d, r, self.rot_dims)
+            qr = step.buffer("latent.qr", (n, T, r + pad), act) if r + pad else None
+            if pad:
+                ops.latent.zero_(qr)
+            ops.latent.latent_q_split(q, self.freq, self.mag, step.positions, qn, qr if r else None, n, d, r, self.rot_dims)
             qa = step.buffer("latent.qa", (n, T, R), act)
             ops.latent.heads_gemm(qn, self.w_uk_t, qa)
             ol = ol.view(n, T, R)
@@ -153,12 +160,16 @@ class LatentAttention(Mixer):
         if fast:
             qa = step.buffer("latent.qa", (T, n * R), act)
             ops.head_gemm(q, d + r, self.w_uk_t, qa, R, n, choices=step.choices)
-            qr = step.buffer("latent.qr", (T, n * r), act) if r else None
+            qr = step.buffer("latent.qr", (T, n * (r + pad)), act) if r + pad else None
+            if pad:
+                ops.latent.zero_(qr)
             if r:
                 ops.latent_q_rotate(q, self.freq, self.mag, step.positions, qr, n, d, r, self.rot_dims, 0)
             ops.latent.latent_attention_mfma(qa, qr, rows, ol, step, table, n, R, self.scale, self.window, head_major=False)
         else:
             qp = step.buffer("latent.qp", (T, n * D), act)
+            if pad:
+                ops.latent.zero_(qp)
             ops.head_gemm(q, d + r, self.w_uk_t, qp, D, n, choices=step.choices)
             if r:
                 ops.latent_q_rotate(q, self.freq, self.mag, step.positions, qp, n, d, r, self.rot_dims, R)

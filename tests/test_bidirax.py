@@ -170,7 +170,7 @@ def test_config_reader_names_and_cache_specs():
     assert [c.cache_id for c in model.schedule] == [0, 1, 2, 1, 4] and not model.schedule[3].write_cache
     for path, value, text in [(("layers", 1, "mixer", "mask"), None, "mask"), (("layers", 3, "mixer", "kv_from"), 3, "earlier"),
                               (("layers", 0, "type"), "attention", "none of"), (("layers", 0, "mixer", "rot", "dims"), 10, "dims"),
-                              (("layers", 1, "mlp", "router", "top"), 9, "top"), (("layers", 3, "mixer", "kv_rank"), 16, "kv_rank"),
+                              (("layers", 1, "mlp", "router", "top"), 9, "top"), (("layers", 3, "mixer", "kv_rank"), 16, "kv_rank"), (("layers", 3, "mixer", "rot_dim"), 4, "rot"),
                               (("norm",), None, "norm")]:
         bad = copy.deepcopy(bm.MIXED)
         at = bad

@@ -78,6 +78,8 @@ ONE_LAYER = {
                                                  bm.windowed(heads=3, dim=6, vdim=4, window=11, kv_from=0, sharp=4.0, mlp=None)]),
     "reads_the_layer_in_front_narrower": bm.config([bm.windowed(window=12, sharp=4.0, mlp=None),
                                                     bm.windowed(heads=1, dim=14, vdim=10, window=3, kv_from=0, sharp=4.0, mlp=None)]),
+    "reads_a_rotated_layers_latent": bm.config([bm.rotated(heads=2, dim=8, rot_dim=6, vdim=8, kv_rank=12, sharp=3.0, mlp=None),
+                                                bm.windowed(heads=3, dim=6, vdim=4, kv_rank=12, window=30, kv_from=0, sharp=4.0, mlp=None)]),
     "dense": bm.config([bm.windowed(mlp="dense")], embed_scale=1.0),
     "experts_and_shared": bm.config([bm.windowed(mlp="moe")]),
     "experts_alone_top_one": bm.config([bm.windowed(mlp=bm.feed_forward("moe", experts=3, top=1, scale=1.0, shared=None))]),
@@ -133,6 +135,42 @@ def test_every_schedule_gives_the_plain_logits(tmp_path, cfg_name, dtype):
                 first = first or _stacked(got)
                 assert _most(got, first) < BF16_BETWEEN_SCHEDULES and _mean(got, first) < BF16_BETWEEN_SCHEDULES / 2, (what, page)
             assert not cache.manager.live_requests()
+
+
+MATRIX_CORES = {
+    # three heads (a wavefront's 16 rows are 5 tokens and a third), unrotated entries no multiple of 8 (the per-head maps
+    # stay plain), a window that ends inside blocks of rows
+    "three_heads": bm.config([bm.rotated(heads=3, dim=12, rot_dim=32, vdim=10, kv_rank=32, q_rank=24, sharp=3.0, mlp=None),
+                              bm.windowed(heads=3, dim=12, vdim=10, kv_rank=64, q_rank=24, window=37, sharp=3.0, mlp=None)], width=32),
+    # 80 heads (two workgroups a token), a latent of 16, a reader without rotation over rotated rows
+    "eighty_heads": bm.config([bm.rotated(heads=80, dim=8, rot_dim=16, vdim=8, kv_rank=16, q_rank=16, sharp=2.0, mlp=None),
+                               bm.windowed(heads=5, dim=16, vdim=8, kv_rank=16, q_rank=16, window=50, kv_from=0, sharp=3.0, mlp=None)],
+                              width=32),
+    # rows of 320 and a latent of 256 (the second instance of the kernel), 130 tokens a run of keys
+    "wide_rows": bm.config([bm.rotated(heads=4, dim=16, rot_dim=64, vdim=16, kv_rank=256, q_rank=32, sharp=2.0, mlp=None)], width=32),
+    # rows of 576 and a latent of 512 (the third instance)
+    "widest_rows": bm.config([bm.rotated(heads=2, dim=16, rot_dim=64, vdim=16, kv_rank=512, q_rank=32, sharp=2.0, mlp=None)], width=32),
+}
+
+
+@pytest.mark.parametrize("name", sorted(MATRIX_CORES))
+def test_the_matrix_core_attention_at_other_sizes(tmp_path, name):
+    """bfloat16 on the matrix cores against the same model on the plain-precision kernels (what differs is the rounding of
+    the softmax weights and the order of sums), under every schedule, and both against the plain model."""
+    from llmengine.ops import KernelChoices
+    cfg = MATRIX_CORES[name]
+    engine, weights = _engine(tmp_path, cfg, 21, "bf16")
+    slow_engine, _ = _engine(tmp_path / "plain", cfg, 21, "bf16", weights=weights, kernel_choices=KernelChoices(fast_attention=False))
+    V = cfg["vocab"]
+    requests = {"a": _tokens(300, V, 1), "b": _tokens(21, V, 2), "c": _tokens(1, V, 3)}
+    ref = _reference(cfg, weights, requests)
+    slow = _stacked(replay.run_trace(slow_engine, slow_engine.new_cache(32, 16, 3), replay.whole(requests)))
+    for steps in (replay.whole(requests), replay.tail_one_by_one(requests, tail=150), replay.portions(requests, sizes=(33, 2, 64, 7, 1, 41)),
+                  replay.mixed(requests, max_live=3, sizes=(50, 3, 24, 2), seed=4)):
+        got = replay.run_trace(engine, engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3), steps)
+        assert _covered(got, requests)
+        assert _mean(got, slow) < 1e-2 and _most(got, slow) < 3e-2
+        assert _mean(got, ref) < 6e-2
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
